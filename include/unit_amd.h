@@ -1,0 +1,150 @@
+/*
+ * unit_amd -- C ABI of the MI355X (gfx950) tensorized conv2d / dense / GEMM path.
+ *
+ * The reference has no FFI of its own: its operators are Python functions on TVM
+ * tensors.  Each entry point below names the reference operator (file:line, relative to
+ * the reference tree) whose arithmetic it replaces; a binding only has to pass device
+ * pointers and the operator's own shape arguments.
+ *
+ * Conventions
+ *   - every pointer is a device pointer owned by the caller; the library never
+ *     allocates or frees device memory and keeps no state between calls;
+ *   - `stream` is a hipStream_t (NULL = default stream); calls enqueue work and return
+ *     without synchronising;
+ *   - return value 0 = enqueued; <0 = rejected (UNIT_E_*), nothing enqueued, and
+ *     unit_last_error() returns a thread-local message;
+ *   - int8 results are exact (int32 accumulation, wrapping mod 2^32 like vpdpbusd);
+ *     fp16 inputs are multiplied and accumulated in fp32 on the MFMA unit;
+ *   - a tensor may not exceed 2^31-1 bytes.
+ */
+#ifndef UNIT_AMD_H
+#define UNIT_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define UNIT_OK 0
+#define UNIT_E_ARG (-1)     /* bad shape / null pointer / unsupported combination */
+#define UNIT_E_LAUNCH (-2)  /* HIP refused the launch */
+#define UNIT_E_DEVICE (-3)  /* current device is not gfx950 */
+
+typedef void *unit_stream_t;
+
+/* ABI version (major * 100 + minor). */
+int unit_version(void);
+/* Message for the last non-zero return on this thread ("" if none). */
+const char *unit_last_error(void);
+/* Name of the kernel variant the last successful compute call on this thread enqueued
+ * (e.g. "i8conv_x256_y256_k128_w8"): the analogue of the tuned-schedule index the reference
+ * logs per shape (python/tensorizer/tune.py:20-31). */
+const char *unit_last_variant(void);
+
+/* Geometry of one 2-D convolution; C and K are the channel counts as stored in the blocked
+ * tensors (already rounded up: C % cb == 0, K % 16 == 0, apps/cpu/kernel/conv2d.py:18-22). */
+typedef struct unit_conv_desc {
+  int32_t N, C, H, W; /* data: batch, input channels, height, width (unpadded) */
+  int32_t K, KH, KW;  /* output channels, kernel height, width */
+  int32_t sh, sw;     /* strides */
+  int32_t pt, pl, pb, pr; /* zero padding: top, left, bottom, right */
+  int32_t dh, dw;     /* dilation */
+  int32_t cb;         /* input-channel block of the data layout: 16 or 4 (int8); 16 (fp16) */
+} unit_conv_desc;
+
+/* Output height/width for a descriptor; UNIT_E_ARG if the window does not fit. */
+int unit_conv_out_hw(const unit_conv_desc *d, int32_t *OH, int32_t *OW);
+
+/* ------------------------------------------------------------------ int8 compute */
+
+/* topi.nn.conv2d_NCHWc_int8(data, kernel, stride, padding, dilation, out_dtype='int32',
+ * layout='NCHW{cb}c', out_layout='NCHW16c') as called at apps/cpu/kernel/conv2d.py:50-51
+ * (closed form: apps/cpu/kernel/conv3d.py:60-64).
+ *   data   u8  (N, C/cb, H, W, cb)
+ *   weight s8  (K/16, C/cb, KH, KW, cb/4, 16, 4)       -- the reference's VNNI pre-pack
+ *   out    i32 (N, K/16, OH, OW, 16)
+ * u8 x s8 -> i32, replacing llvm.x86.avx512.vpdpbusd.512
+ * (python/tensorizer/intrinsics/cpu.py:42-49,189-193) with v_mfma_i32_32x32x32_i8. */
+int unit_conv2d_nchwc_u8s8s32(const unit_conv_desc *d, const void *data, const void *weight,
+                              void *out, unit_stream_t stream);
+
+/* topi.x86.dense_dotprod(data, weight, None, 'int32') as called at
+ * apps/cpu/kernel/int8-gemm.py:13-16.
+ *   a   u8  (M, K) row-major
+ *   wp  s8  (N/128, K/4, 128, 4),  wp[n/128][k/4][n%128][k%4] = W[n][k]
+ *   c   i32 (M, N) = a . W^T
+ * N % 128 == 0, K % 16 == 0. */
+int unit_dense_dotprod_u8s8s32(const void *a, const void *wp, void *c, int32_t M, int32_t N,
+                               int32_t K, unit_stream_t stream);
+
+/* relay.nn.dense(x, w, out_dtype='int32') of apps/cpu/relay/int8-gemm.py:14-16 on the
+ * un-packed weight:  a u8 (M, K), w s8 (N, K) row-major, c i32 (M, N) = a . w^T.
+ * K % 16 == 0. */
+int unit_dense_u8s8s32(const void *a, const void *w, void *c, int32_t M, int32_t N, int32_t K,
+                       unit_stream_t stream);
+
+/* ------------------------------------------------------------------ fp16 compute */
+
+/* The fp16 GEMM of apps/gpu/gemm.py:8-20 (CUDA form: poc/tensorcore/gemm-prefetch.cu:66-164):
+ *   c[x][y] = sum_k f32(a[x][k]) * f32(b[k][y]),  a f16 (M, K), b f16 (K, N), row-major;
+ * c is f32 when out_f16 == 0, else f16 (round-to-nearest-even of the fp32 sum).
+ * K % 8 == 0, N % 4 == 0.  Replaces wmma.m16n16k16 (python/tensorizer/intrinsics/gpu.py:104-216)
+ * with v_mfma_f32_32x32x16_f16. */
+int unit_gemm_f16(const void *a, const void *b, void *c, int32_t M, int32_t N, int32_t K,
+                  int32_t out_f16, unit_stream_t stream);
+
+/* _conv2d_NCHW16c_OHWI16o_impl(a, b, stride_h, stride_w, out_type)
+ * (python/tensorizer/ops/gpu.py:8-53) on packed operands:
+ *   a   f16 (N, C/16, H, W, 16)
+ *   b   f16 (K/16, C/16, KH, KW, 16 in, 16 out)
+ *   out f32 (N, K/16, OH, OW, 16)
+ * Valid convolution: the descriptor's padding must be 0 and dilation 1, cb == 16 (the
+ * reference operator has no padding argument; callers pre-pad). */
+int unit_conv2d_nchw16c_f16f32(const unit_conv_desc *d, const void *a, const void *b, void *out,
+                               unit_stream_t stream);
+
+/* ------------------------------------------------------------------ layout / pre-pack */
+
+/* layout_transform NCHW -> NCHW{cb}c (apps/cpu/relay/result.log:7,6807-6808; in-op form
+ * python/tensorizer/ops/gpu.py:26-28): dst[n][ci][h][w][c] = src[n][cb*ci+c][h][w], zero for
+ * cb*ci+c >= C.  elem_size is the element width in bytes (1, 2 or 4). */
+int unit_pack_nchwc(const void *src, void *dst, int32_t N, int32_t C, int32_t H, int32_t W,
+                    int32_t cb, int32_t elem_size, unit_stream_t stream);
+
+/* layout_transform NCHW{cb}c -> NCHW (apps/cpu/relay/result.log:25), keeping the first C
+ * channels of the ceil(C/cb) blocks. */
+int unit_unpack_nchwc(const void *src, void *dst, int32_t N, int32_t C, int32_t H, int32_t W,
+                      int32_t cb, int32_t elem_size, unit_stream_t stream);
+
+/* int8 conv weight pre-pack OIHW -> (ceil(O/16), ceil(I/cb), KH, KW, cb/4, 16, 4): the
+ * transpose/reshape chain of apps/cpu/relay/result.log:8-13 (cb = 16) and :6809-6815
+ * (cb = 4, input channels zero-padded);  dst[ko][ci][kh][kw][e][kb][i] =
+ * src[16ko+kb][cb*ci+4e+i][kh][kw], zero outside O x I. */
+int unit_prepack_conv_weight_s8(const void *src, void *dst, int32_t O, int32_t I, int32_t KH,
+                                int32_t KW, int32_t cb, unit_stream_t stream);
+
+/* int8 dense weight pre-pack (N, K) -> (N/128, K/4, 128, 4) (placeholder shape at
+ * apps/cpu/kernel/int8-gemm.py:14; 16x4 analogue poc/vnni/vnni_dense.py:10-11). */
+int unit_prepack_dense_weight_s8(const void *src, void *dst, int32_t N, int32_t K,
+                                 unit_stream_t stream);
+
+/* fp16 conv weight pack OIHW -> (O/16, I/16, KH, KW, 16 in, 16 out)
+ * (python/tensorizer/ops/gpu.py:29-31).  O % 16 == 0, I % 16 == 0. */
+int unit_prepack_conv_weight_f16(const void *src, void *dst, int32_t O, int32_t I, int32_t KH,
+                                 int32_t KW, unit_stream_t stream);
+
+/* ------------------------------------------------------------------ diagnostics */
+
+/* One v_mfma_i32_32x32x32_i8 / v_mfma_f32_32x32x16_f16 on a single wavefront, operands and
+ * result in plain row-major form:  a (32, 32) s8 | f16 (32, 16);  b (32 cols, 32) s8 |
+ * (32 cols, 16) f16 given K-contiguous per column;  c (32, 32) i32 | f32 = a . b^T.
+ * The counterpart of poc/vnni/poc.cc:17-38 (instruction-semantics check). */
+int unit_mfma_tile_i8(const void *a, const void *b, void *c, unit_stream_t stream);
+int unit_mfma_tile_f16(const void *a, const void *b, void *c, unit_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* UNIT_AMD_H */

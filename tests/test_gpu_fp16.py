@@ -1,0 +1,94 @@
+"""Parity of the fp16 HIP path against a float64 reference on the fp16-rounded inputs.
+Tolerance (BASELINE north star): max |d| / max(|ref|, eps * max|ref|) <= 1e-2."""
+import numpy as np
+import pytest
+import torch
+
+import unit_amd as U
+from unit_amd import rng
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-2
+
+
+def _t(a, dev):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def max_rel(out, ref):
+    ref = np.asarray(ref, dtype=np.float64)
+    floor = 1e-3 * np.abs(ref).max()
+    return float((np.abs(out.astype(np.float64) - ref) / np.maximum(np.abs(ref), floor)).max())
+
+
+def test_mfma_tile_f16_lane_layout(dev):
+    import ctypes
+    from unit_amd import _lib
+    a = (rng.uniform_s8((32, 16), 1) % 5).astype(np.float16)
+    b = (rng.uniform_s8((32, 16), 2) % 7).astype(np.float16)
+    ta, tb = _t(a, dev), _t(b, dev)
+    tc = torch.zeros((32, 32), dtype=torch.float32, device=dev)
+    _lib.check(_lib.load().unit_mfma_tile_f16(ta.data_ptr(), tb.data_ptr(), tc.data_ptr(), None))
+    torch.cuda.synchronize()
+    assert np.array_equal(tc.cpu().numpy(), (a.astype(np.float64) @ b.astype(np.float64).T).astype(np.float32))
+
+
+GEMM_CASES = [(128, 768, 3072), (32, 32, 64), (100, 132, 72), (512, 4096, 256), (4096, 2048, 512), (2050, 4100, 136)]
+
+
+@pytest.mark.parametrize("M,N,K", GEMM_CASES)
+@pytest.mark.parametrize("out_dtype", ["float32", "float16"])
+def test_gemm_fp16(dev, oracle, M, N, K, out_dtype):
+    a = rng.normal_f16((M, K), 31 + M, 1.0 / np.sqrt(K))
+    b = rng.normal_f16((K, N), 57 + N)
+    out = U.gemm_fp16(_t(a, dev), _t(b, dev), out_dtype)
+    torch.cuda.synchronize()
+    ref = oracle.gemm_f16(a, b)
+    err = max_rel(out.cpu().numpy(), ref)
+    assert err <= (REL_TOL if out_dtype == "float32" else REL_TOL), (err, U.last_variant())
+
+
+def test_gemm_fp16_integer_exact(dev, oracle):
+    """Small-integer operands (the arange % 7 recipe of apps/gpu/conv-wdim.py:33-36) make every
+    fp32 partial sum exact, so the result must match the float64 reference bit for bit."""
+    M, N, K = 256, 384, 512
+    a = (np.arange(M * K).reshape(M, K) % 7).astype(np.float16)
+    b = (np.arange(K * N).reshape(K, N) % 5 - 2).astype(np.float16)
+    out = U.gemm_fp16(_t(a, dev), _t(b, dev)).cpu().numpy()
+    assert np.array_equal(out.astype(np.float64), oracle.gemm_f16(a, b))
+
+
+CONV_CASES = [
+    # N, C, H, W, K, kernel, stride
+    (1, 64, 16, 18, 64, 3, 1),     # apps/gpu/conv-wdim.py shape family
+    (1, 16, 9, 9, 16, 1, 1),
+    (2, 32, 12, 10, 48, 3, 2),
+    (1, 256, 30, 30, 256, 3, 2),   # gpu-tune.log:27-28
+    (1, 256, 56, 56, 128, 1, 1),   # gpu-tune.log:5-6
+    (4, 128, 30, 30, 128, 3, 1),
+    (32, 256, 16, 16, 256, 3, 1),  # batch 32, 256-channel tile
+]
+
+
+@pytest.mark.parametrize("N,C,H,W,K,ks,stride", CONV_CASES)
+def test_conv2d_fp16(dev, oracle, N, C, H, W, K, ks, stride):
+    a = rng.normal_f16((N, C // 16, H, W, 16), 5 + C)
+    b = rng.normal_f16((K // 16, C // 16, ks, ks, 16, 16), 9 + K, 1.0 / np.sqrt(C * ks * ks))
+    out = U.conv2d_NCHW16c_OHWI16o(_t(a, dev), _t(b, dev), stride, stride, "float32")
+    torch.cuda.synchronize()
+    ref = oracle.conv2d_nchw16c_f16(a, b, stride, stride)
+    assert tuple(out.shape) == ref.shape
+    err = max_rel(out.cpu().numpy(), ref)
+    assert err <= REL_TOL, (err, U.last_variant())
+
+
+def test_conv2d_fp16_unpacked_operands(dev, oracle):
+    """4-D NCHW + OIHW operands are packed in-op like python/tensorizer/ops/gpu.py:25-33; integer
+    data makes the comparison exact."""
+    N, C, H, W, K = 1, 32, 10, 10, 32
+    a = (np.arange(N * C * H * W).reshape(N, C, H, W) % 7).astype(np.float16)
+    b = (np.arange(K * C * 9).reshape(K, C, 3, 3) % 5 - 2).astype(np.float16)
+    out = U.conv2d_NCHW16c_OHWI16o(_t(a, dev), _t(b, dev), 1, 1).cpu().numpy()
+    ref = oracle.conv2d_nchw16c_f16(oracle.pack_nchwc(a, 16), oracle.prepack_conv_weight_f16(b), 1, 1)
+    assert np.array_equal(out.astype(np.float64), ref)

@@ -1,0 +1,113 @@
+"""Parity of the int8 HIP path (through the C ABI) against the CPU oracle: bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+import unit_amd as U
+from unit_amd import rng
+
+pytestmark = pytest.mark.gpu
+
+
+def _t(a, dev):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def test_mfma_tile_i8_lane_layout(dev):
+    """One v_mfma_i32_32x32x32_i8 against the integer matrix product: pins the operand / result
+    lane mapping every kernel relies on (the counterpart of the vpdpbusd known-answer program)."""
+    import ctypes
+    from unit_amd import _lib
+    a = rng.uniform_s8((32, 32), 11)
+    b = rng.uniform_s8((32, 32), 12)
+    ta, tb = _t(a, dev), _t(b, dev)
+    tc = torch.zeros((32, 32), dtype=torch.int32, device=dev)
+    _lib.check(_lib.load().unit_mfma_tile_i8(ta.data_ptr(), tb.data_ptr(), tc.data_ptr(), None))
+    torch.cuda.synchronize()
+    ref = a.astype(np.int64) @ b.astype(np.int64).T
+    assert np.array_equal(tc.cpu().numpy(), ref.astype(np.int32))
+
+
+DENSE_CASES = [
+    # M, N, K
+    (1, 128, 16),          # the reference's M=1 dense (cpu-shapes.log:367) in miniature
+    (1, 1024, 512),        # resnet18 classifier: (1, 512) x (8, 128, 128, 4)
+    (128, 3072, 768),      # apps/cpu/kernel/int8-gemm.py:9
+    (37, 256, 80),         # ragged M, K not a multiple of the stage
+    (300, 384, 272),
+    (4096, 2048, 256),     # large-tile variant (128 workgroups of 256x256)
+    (2100, 4096, 144),     # large tiles with a ragged M edge and a K tail
+]
+
+
+@pytest.mark.parametrize("M,N,K", DENSE_CASES)
+@pytest.mark.parametrize("packed", [True, False])
+def test_dense_bit_exact(dev, oracle, M, N, K, packed):
+    a = rng.uniform_u8((M, K), 100 + M)
+    w = rng.uniform_s8((N, K), 200 + N)
+    wp = oracle.prepack_dense_weight(w)
+    ref = oracle.c_dense(a, wp)
+    if M * N * K <= 1 << 24:
+        assert np.array_equal(ref, oracle.dense_logical(a, w))
+    out = U.dense_dotprod(_t(a, dev), _t(wp if packed else w, dev))
+    torch.cuda.synchronize()
+    assert out.dtype == torch.int32 and tuple(out.shape) == (M, N)
+    assert np.array_equal(out.cpu().numpy(), ref), U.last_variant()
+
+
+def test_dense_extremes(dev, oracle):
+    """255 x -128 everywhere: the largest negative accumulation (K * -32640), and 255 x 127."""
+    M, N, K = 64, 128, 4096
+    a = np.full((M, K), 255, dtype=np.uint8)
+    for val in (-128, 127):
+        w = np.full((N, K), val, dtype=np.int8)
+        out = U.dense(_t(a, dev), _t(w, dev)).cpu().numpy()
+        assert (out == 255 * val * K).all()
+    # zeros stay zero (the u8 -> s8 shift and its correction cancel)
+    out = U.dense(_t(np.zeros((M, K), np.uint8), dev), _t(rng.uniform_s8((N, K), 5), dev)).cpu().numpy()
+    assert (out == 0).all()
+
+
+CONV_CASES = [
+    # N, C, H, W, K, kernel, stride, pad, dilation
+    (1, 64, 56, 56, 64, 3, 1, 1, 1),       # BASELINE config (1)
+    (2, 32, 9, 7, 32, 3, 1, 1, 1),         # tiny, ragged pixel count
+    (1, 16, 8, 8, 48, 1, 2, 0, 1),         # 1x1 stride 2, K not a multiple of 32
+    (3, 64, 14, 14, 128, 1, 1, 0, 1),      # 1x1 = GEMM
+    (1, 128, 28, 28, 128, 3, 1, 1, 1),
+    (1, 64, 56, 56, 128, 3, 2, 1, 1),
+    (1, 256, 14, 14, 512, 3, 2, 1, 1),
+    (1, 512, 7, 7, 512, 3, 1, 1, 1),
+    (1, 4, 32, 32, 64, 7, 2, 3, 1),        # NCHW4c stem, small
+    (1, 4, 224, 224, 64, 7, 2, 3, 1),      # NCHW4c stem, full size
+    (2, 8, 11, 13, 16, 3, 1, (0, 1, 2, 1), 1),   # cb = 4 with two channel blocks, asymmetric pad
+    (2, 16, 12, 12, 32, 3, 1, 2, 2),       # dilation 2
+    (1, 48, 10, 10, 80, 5, (2, 1), (2, 0), 1),   # anisotropic stride / pad, 5x5
+    (32, 64, 56, 56, 64, 1, 1, 0, 1),      # batch 32: 64-channel tile, many workgroups
+    (32, 256, 14, 14, 256, 3, 1, 1, 1),    # batch 32: 256-channel tile
+    (32, 128, 28, 28, 128, 3, 1, 1, 1),    # batch 32: 128-channel tile
+    (8, 512, 7, 7, 2048, 1, 1, 0, 1),
+]
+
+
+@pytest.mark.parametrize("N,C,H,W,K,ks,stride,pad,dil", CONV_CASES)
+def test_conv2d_bit_exact(dev, oracle, N, C, H, W, K, ks, stride, pad, dil):
+    cb = 16 if C % 16 == 0 else 4
+    data = rng.uniform_u8((N, C // cb, H, W, cb), 7 * C + H)
+    wt = rng.uniform_s8((K // 16, C // cb, ks, ks, cb // 4, 16, 4), 3 * K + ks)
+    ref = oracle.c_conv2d_nchwc(data, wt, stride, pad, dil)
+    out = U.conv2d_NCHWc_int8(_t(data, dev), _t(wt, dev), stride, pad, dil, "int32", f"NCHW{cb}c", "NCHW16c")
+    torch.cuda.synchronize()
+    assert tuple(out.shape) == ref.shape
+    assert np.array_equal(out.cpu().numpy(), ref), U.last_variant()
+
+
+def test_conv2d_zero_padding_value(dev, oracle):
+    """Padded pixels are u8 zeros: with all-255 data and all-ones weights every output equals
+    255 * (number of in-image taps) * C, which differs between border and interior."""
+    C, H, K = 16, 6, 16
+    data = np.full((1, 1, H, H, 16), 255, dtype=np.uint8)
+    wt = np.ones((1, 1, 3, 3, 4, 16, 4), dtype=np.int8)
+    out = U.conv2d_NCHWc_int8(_t(data, dev), _t(wt, dev), 1, 1).cpu().numpy()
+    assert out[0, 0, 0, 0, 0] == 255 * 4 * C and out[0, 0, 2, 2, 0] == 255 * 9 * C
+    assert np.array_equal(out, oracle.conv2d_nchwc_int8(data, wt, 1, 1))

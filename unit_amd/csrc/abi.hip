@@ -1,0 +1,135 @@
+// C-ABI plumbing: version, thread-local error / variant strings, device check, convolution
+// geometry validation, and the single-instruction MFMA diagnostics.
+#include "host.hpp"
+#include "loaders.hpp"
+
+namespace unit {
+
+char *error_buf() {
+  static thread_local char buf[256] = "";
+  return buf;
+}
+
+char *variant_buf() {
+  static thread_local char buf[96] = "";
+  return buf;
+}
+
+int check_device() {
+  static thread_local int cached_dev = -1;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(UNIT_E_DEVICE, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev == cached_dev) return UNIT_OK;
+  hipDeviceProp_t prop;
+  e = hipGetDeviceProperties(&prop, dev);
+  if (e != hipSuccess) return fail(UNIT_E_DEVICE, "hipGetDeviceProperties: %s", hipGetErrorString(e));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(UNIT_E_DEVICE, "device %d is %s; this library is built for gfx950 only", dev, prop.gcnArchName);
+  cached_dev = dev;
+  return UNIT_OK;
+}
+
+static int out_hw(const unit_conv_desc *d, int *OH, int *OW, const char *what) {
+  if (d->N <= 0 || d->C <= 0 || d->H <= 0 || d->W <= 0 || d->K <= 0 || d->KH <= 0 || d->KW <= 0)
+    return fail(UNIT_E_ARG, "%s: N, C, H, W, K, KH, KW must be positive", what);
+  if (d->sh <= 0 || d->sw <= 0 || d->dh <= 0 || d->dw <= 0)
+    return fail(UNIT_E_ARG, "%s: strides and dilations must be positive", what);
+  if (d->pt < 0 || d->pl < 0 || d->pb < 0 || d->pr < 0) return fail(UNIT_E_ARG, "%s: negative padding", what);
+  const long eh = (long)d->H + d->pt + d->pb - (long)d->dh * (d->KH - 1) - 1;
+  const long ew = (long)d->W + d->pl + d->pr - (long)d->dw * (d->KW - 1) - 1;
+  if (eh < 0 || ew < 0) return fail(UNIT_E_ARG, "%s: kernel window larger than the padded input", what);
+  *OH = (int)(eh / d->sh) + 1;
+  *OW = (int)(ew / d->sw) + 1;
+  return UNIT_OK;
+}
+
+// tapb: bytes one input pixel contributes per tap (u8 cb16: 16, u8 cb4: 4, f16 cb16: 32)
+int conv_geom(const unit_conv_desc *d, int tapb, ConvGeom *g, const char *what) {
+  int OH, OW;
+  if (int rc = out_hw(d, &OH, &OW, what)) return rc;
+  if (d->C % d->cb) return fail(UNIT_E_ARG, "%s: C (%d) must be a multiple of cb (%d)", what, d->C, d->cb);
+  if (d->K % 16) return fail(UNIT_E_ARG, "%s: K (%d) must be a multiple of 16", what, d->K);
+  if (d->H >= 16384 || d->W >= 16384 || (long)d->KH * d->dh >= 16384 || (long)d->KW * d->dw >= 16384)
+    return fail(UNIT_E_ARG, "%s: spatial extent too large", what);
+  const int cc = d->C / d->cb;
+  const size_t img = (size_t)cc * d->H * d->W * tapb;
+  const size_t npix = (size_t)d->N * OH * OW;
+  if (!fits(img * d->N) || npix > kMaxTensorBytes || !fits((size_t)d->K * cc * d->KH * d->KW * tapb))
+    return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
+  g->N = d->N;
+  g->H = d->H;
+  g->W = d->W;
+  g->OH = OH;
+  g->OW = OW;
+  g->KH = d->KH;
+  g->KW = d->KW;
+  g->sh = d->sh;
+  g->sw = d->sw;
+  g->pt = d->pt;
+  g->pl = d->pl;
+  g->dh = d->dh;
+  g->dw = d->dw;
+  g->npix = (int)npix;
+  g->ntaps = cc * d->KH * d->KW;
+  g->ntab = g->ntaps;
+  g->img_bytes = (u32)img;
+  return UNIT_OK;
+}
+
+namespace {
+
+// a (32, 32) s8 row-major, b (32, 32) s8 with row = output column; c (32, 32) i32 = a . b^T
+__global__ __launch_bounds__(64) void mfma_tile_i8(const char *a, const char *b, int *c) {
+  const int l = threadIdx.x, l32 = l & 31, half = l >> 5;
+  v4i x = *reinterpret_cast<const v4i *>(a + l32 * 32 + half * 16);
+  v4i y = *reinterpret_cast<const v4i *>(b + l32 * 32 + half * 16);
+  v16i acc;
+  for (int r = 0; r < 16; ++r) acc[r] = 0;
+  acc = OpI8::mma(x, y, acc);
+  for (int r = 0; r < 16; ++r) c[(8 * (r >> 2) + 4 * half + (r & 3)) * 32 + l32] = acc[r];
+}
+
+__global__ __launch_bounds__(64) void mfma_tile_f16(const char *a, const char *b, float *c) {
+  const int l = threadIdx.x, l32 = l & 31, half = l >> 5;
+  v4i x = *reinterpret_cast<const v4i *>(a + l32 * 32 + half * 16);
+  v4i y = *reinterpret_cast<const v4i *>(b + l32 * 32 + half * 16);
+  v16f acc;
+  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+  acc = OpF16::mma(x, y, acc);
+  for (int r = 0; r < 16; ++r) c[(8 * (r >> 2) + 4 * half + (r & 3)) * 32 + l32] = acc[r];
+}
+
+}  // namespace
+}  // namespace unit
+
+extern "C" int unit_version(void) { return 100; }
+
+extern "C" const char *unit_last_error(void) { return unit::error_buf(); }
+
+extern "C" const char *unit_last_variant(void) { return unit::variant_buf(); }
+
+extern "C" int unit_conv_out_hw(const unit_conv_desc *d, int32_t *OH, int32_t *OW) {
+  if (!d || !OH || !OW) return unit::fail(UNIT_E_ARG, "unit_conv_out_hw: null pointer");
+  return unit::out_hw(d, OH, OW, "unit_conv_out_hw");
+}
+
+extern "C" int unit_mfma_tile_i8(const void *a, const void *b, void *c, unit_stream_t stream) {
+  using namespace unit;
+  if (!a || !b || !c) return fail(UNIT_E_ARG, "unit_mfma_tile_i8: null pointer");
+  if (int rc = check_device()) return rc;
+  hipLaunchKernelGGL(mfma_tile_i8, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const char *>(a), static_cast<const char *>(b), static_cast<int *>(c));
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "unit_mfma_tile_i8: %s", hipGetErrorString(e));
+}
+
+extern "C" int unit_mfma_tile_f16(const void *a, const void *b, void *c, unit_stream_t stream) {
+  using namespace unit;
+  if (!a || !b || !c) return fail(UNIT_E_ARG, "unit_mfma_tile_f16: null pointer");
+  if (int rc = check_device()) return rc;
+  hipLaunchKernelGGL(mfma_tile_f16, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const char *>(a), static_cast<const char *>(b), static_cast<float *>(c));
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "unit_mfma_tile_f16: %s", hipGetErrorString(e));
+}

@@ -1,0 +1,57 @@
+// int8 dense: c (M, N) i32 = a (M, K) u8 . W^T, W s8 given row-major (N, K) or in the reference's
+// (N/128, K/4, 128, 4) pre-pack.  X operand = a (rows m), Y operand = W (rows n).
+#include "epilogues.hpp"
+#include "host.hpp"
+#include "loaders.hpp"
+
+namespace unit {
+namespace {
+
+template <class T, bool PACKED>
+int run_dense(const void *a, const void *w, void *c, int M, int N, int K, hipStream_t s) {
+  using XL = RowMajorLoader<T::BX, T::BKB, T::NT, true>;
+  using YLrm = RowMajorLoader<T::BY, T::BKB, T::NT, false>;
+  using YLpk = VnniLoader<T::BY, T::BKB, T::NT, 128>;
+  using Epi = GemmEpilogue<OpI8, false>;
+  typename XL::Params xp{static_cast<const char *>(a), M, K, K};
+  typename Epi::Params ep{c, M, N};
+  const int nk = ceil_div(K, T::BKB), gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
+  set_variant("i8dense%s_x%d_y%d_k%d_w%d", PACKED ? "pk" : "rm", T::BX, T::BY, T::BKB, T::NT / 64);
+  if constexpr (PACKED) {
+    typename YLpk::Params yp{static_cast<const char *>(w), N, K / 4};
+    return launch_mma<OpI8, T, XL, YLpk, Epi, WS_Y>(xp, yp, ep, nk, gx, gy, 4, 0, s, "dense_dotprod");
+  } else {
+    typename YLrm::Params yp{static_cast<const char *>(w), N, K, K};
+    return launch_mma<OpI8, T, XL, YLrm, Epi, WS_Y>(xp, yp, ep, nk, gx, gy, 4, 0, s, "dense");
+  }
+}
+
+template <bool PACKED>
+int dense(const void *a, const void *w, void *c, int M, int N, int K, unit_stream_t stream) {
+  const char *what = PACKED ? "unit_dense_dotprod_u8s8s32" : "unit_dense_u8s8s32";
+  if (!a || !w || !c) return fail(UNIT_E_ARG, "%s: null pointer", what);
+  if (M <= 0 || N <= 0 || K <= 0) return fail(UNIT_E_ARG, "%s: M, N, K must be positive (got %d, %d, %d)", what, M, N, K);
+  if (K % 16) return fail(UNIT_E_ARG, "%s: K must be a multiple of 16 (got %d)", what, K);
+  if (PACKED && N % 128) return fail(UNIT_E_ARG, "%s: N must be a multiple of 128 (got %d)", what, N);
+  if (!PACKED && N % 4) return fail(UNIT_E_ARG, "%s: N must be a multiple of 4 (got %d)", what, N);
+  if (!fits((size_t)M * K) || !fits((size_t)N * K) || !fits((size_t)M * N * 4))
+    return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
+  if (int rc = check_device()) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const long tiles_big = (long)ceil_div(M, 256) * ceil_div(N, 256);
+  if (M >= 256 && N >= 256 && tiles_big >= 128) return run_dense<Tile<256, 256, 128, 2, 4>, PACKED>(a, w, c, M, N, K, s);
+  return run_dense<Tile<128, 128, 64, 2, 2>, PACKED>(a, w, c, M, N, K, s);
+}
+
+}  // namespace
+}  // namespace unit
+
+extern "C" int unit_dense_dotprod_u8s8s32(const void *a, const void *wp, void *c, int32_t M, int32_t N, int32_t K,
+                                          unit_stream_t stream) {
+  return unit::dense<true>(a, wp, c, M, N, K, stream);
+}
+
+extern "C" int unit_dense_u8s8s32(const void *a, const void *w, void *c, int32_t M, int32_t N, int32_t K,
+                                  unit_stream_t stream) {
+  return unit::dense<false>(a, w, c, M, N, K, stream);
+}

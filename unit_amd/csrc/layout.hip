@@ -1,0 +1,245 @@
+// Layout transforms and weight pre-packs.  All are pure byte permutations bound by HBM traffic
+// (read once + write once); none touches the MFMA unit.
+#include "host.hpp"
+
+namespace unit {
+namespace {
+
+// ---- NCHW <-> NCHW{CB}c -------------------------------------------------------------------
+// A thread moves PP = 4 / ES consecutive pixels of one channel block: CB 4-byte words (one per
+// channel plane, coalesced across lanes) <-> PP contiguous rows of CB elements.
+template <int ES, int CB, bool PACK>
+__global__ __launch_bounds__(256) void nchwc_words(const char *src, char *dst, int C, int HW, int cc,
+                                                   int groups /* HW / PP */) {
+  constexpr int PP = 4 / ES, ROWW = CB * ES / 4;  // words per output row
+  const int g = blockIdx.x * 256 + threadIdx.x;
+  if (g >= groups) return;
+  const int plane = blockIdx.y;  // n * cc + ci
+  const int n = plane / cc, ci = plane - n * cc;
+  const size_t p0 = (size_t)g * PP;
+  const char *nchw = PACK ? src : dst;
+  u32 w[CB];
+  u32 rows[PP][ROWW];
+  if (PACK) {
+#pragma unroll
+    for (int c = 0; c < CB; ++c) {
+      const int ch = ci * CB + c;
+      w[c] = ch < C ? *reinterpret_cast<const u32 *>(nchw + (((size_t)n * C + ch) * HW + p0) * ES) : 0u;
+    }
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp)
+#pragma unroll
+      for (int j = 0; j < ROWW; ++j) {
+        u32 v = 0;
+#pragma unroll
+        for (int e = 0; e < 4 / ES; ++e) {
+          const u32 el = ES == 4 ? w[j] : (w[j * (4 / ES) + e] >> (8 * ES * pp)) & (ES == 1 ? 0xffu : 0xffffu);
+          v |= el << (8 * ES * e);
+        }
+        rows[pp][j] = v;
+      }
+    char *o = dst + ((size_t)plane * HW + p0) * CB * ES;
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp)
+#pragma unroll
+      for (int j = 0; j < ROWW; ++j) reinterpret_cast<u32 *>(o)[pp * ROWW + j] = rows[pp][j];
+  } else {
+    const char *in = src + ((size_t)plane * HW + p0) * CB * ES;
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp)
+#pragma unroll
+      for (int j = 0; j < ROWW; ++j) rows[pp][j] = reinterpret_cast<const u32 *>(in)[pp * ROWW + j];
+#pragma unroll
+    for (int c = 0; c < CB; ++c) {
+      u32 v = 0;
+#pragma unroll
+      for (int pp = 0; pp < PP; ++pp) {
+        const u32 word = rows[pp][c * ES / 4];
+        const u32 el = ES == 4 ? word : (word >> (8 * ES * (c % (4 / ES)))) & (ES == 1 ? 0xffu : 0xffffu);
+        v |= el << (8 * ES * pp);
+      }
+      const int ch = ci * CB + c;
+      if (ch < C) *reinterpret_cast<u32 *>(dst + (((size_t)n * C + ch) * HW + p0) * ES) = v;
+    }
+  }
+}
+
+// any shape / element size: one thread per blocked element
+template <bool PACK>
+__global__ __launch_bounds__(256) void nchwc_elems(const char *src, char *dst, int C, int HW, int cc, int cb,
+                                                   int es, size_t total) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int c = (int)(i % cb);
+  const size_t r = i / cb;
+  const size_t p = r % HW, plane = r / HW;
+  const int ci = (int)(plane % cc);
+  const size_t n = plane / cc;
+  const int ch = ci * cb + c;
+  const size_t flat = ((n * C + ch) * HW + p) * es;
+  for (int b = 0; b < es; ++b) {
+    if (PACK)
+      dst[i * es + b] = ch < C ? src[flat + b] : 0;
+    else if (ch < C)
+      dst[flat + b] = src[i * es + b];
+  }
+}
+
+template <bool PACK>
+int nchwc(const void *src, void *dst, int N, int C, int H, int W, int cb, int es, hipStream_t s, const char *what) {
+  if (!src || !dst) return fail(UNIT_E_ARG, "%s: null pointer", what);
+  if (N <= 0 || C <= 0 || H <= 0 || W <= 0) return fail(UNIT_E_ARG, "%s: N, C, H, W must be positive", what);
+  if (cb <= 0 || cb > 64) return fail(UNIT_E_ARG, "%s: cb must be in 1..64 (got %d)", what, cb);
+  if (es != 1 && es != 2 && es != 4) return fail(UNIT_E_ARG, "%s: elem_size must be 1, 2 or 4 (got %d)", what, es);
+  const int cc = ceil_div(C, cb);
+  const size_t hw = (size_t)H * W, total = (size_t)N * cc * hw * cb;
+  if (!fits(total * es)) return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
+  if (int rc = check_device()) return rc;
+  const char *in = static_cast<const char *>(src);
+  char *out = static_cast<char *>(dst);
+  const int HW = (int)hw, pp = 4 / es;
+  const bool words = HW % pp == 0 && (cb == 16 || (cb == 4 && es == 1)) && (size_t)N * cc <= 65535;
+  if (words) {
+    const int groups = HW / pp;
+    dim3 grid(ceil_div(groups, 256), N * cc);
+#define UNIT_NCHWC(ES, CB)                                                                                   \
+  hipLaunchKernelGGL((nchwc_words<ES, CB, PACK>), grid, dim3(256), 0, s, in, out, C, HW, cc, groups)
+    if (es == 1 && cb == 16) UNIT_NCHWC(1, 16);
+    else if (es == 1 && cb == 4) UNIT_NCHWC(1, 4);
+    else if (es == 2) UNIT_NCHWC(2, 16);
+    else UNIT_NCHWC(4, 16);
+#undef UNIT_NCHWC
+  } else {
+    hipLaunchKernelGGL(nchwc_elems<PACK>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, in, out, C, HW,
+                       cc, cb, es, total);
+  }
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+}
+
+// ---- weight pre-packs ---------------------------------------------------------------------
+// dst[ko][ci][kh][kw][e][kb][i] = src[16ko+kb][cb*ci+4e+i][kh][kw]; one thread per dst dword
+__global__ __launch_bounds__(256) void prepack_conv_s8(const signed char *src, int *dst, int O, int I, int KH,
+                                                       int KW, int cb, int cc, size_t words) {
+  const size_t wi = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (wi >= words) return;
+  const int E = cb / 4;
+  size_t r = wi;
+  const int kb = (int)(r % 16);
+  r /= 16;
+  const int e = (int)(r % E);
+  r /= E;
+  const int kw = (int)(r % KW);
+  r /= KW;
+  const int kh = (int)(r % KH);
+  r /= KH;
+  const int ci = (int)(r % cc);
+  const int ko = (int)(r / cc);
+  const int o = 16 * ko + kb;
+  u32 v = 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int ic = cb * ci + 4 * e + i;
+    if (o < O && ic < I) v |= (u32)(unsigned char)src[(((size_t)o * I + ic) * KH + kh) * KW + kw] << (8 * i);
+  }
+  dst[wi] = (int)v;
+}
+
+// dst[n/128][k/4][n%128][k%4] = src[n][k]; one thread per dword; a 128-thread row of the block
+// reads 128 different rows n at the same k/4: 4-byte reads with stride K (served by L2), and
+// writes 512 contiguous bytes
+__global__ __launch_bounds__(256) void prepack_dense_s8(const int *src, int *dst, int K4, size_t words) {
+  const size_t wi = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (wi >= words) return;
+  const int nl = (int)(wi % 128);
+  const size_t r = wi / 128;
+  const int kg = (int)(r % K4);
+  const size_t nb = r / K4;
+  dst[wi] = src[(nb * 128 + nl) * K4 + kg];
+}
+
+// dst[oc][ic][x][y][ib][ob] = src[16oc+ob][16ic+ib][x][y]; one thread per element
+__global__ __launch_bounds__(256) void prepack_conv_f16(const unsigned short *src, unsigned short *dst, int I,
+                                                        int KH, int KW, size_t total) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  size_t r = i;
+  const int ob = (int)(r % 16);
+  r /= 16;
+  const int ib = (int)(r % 16);
+  r /= 16;
+  const int y = (int)(r % KW);
+  r /= KW;
+  const int x = (int)(r % KH);
+  r /= KH;
+  const int ic = (int)(r % (I / 16));
+  const int oc = (int)(r / (I / 16));
+  dst[i] = src[(((size_t)(16 * oc + ob) * I + 16 * ic + ib) * KH + x) * KW + y];
+}
+
+int launched(const char *what) {
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+}
+
+}  // namespace
+}  // namespace unit
+
+extern "C" int unit_pack_nchwc(const void *src, void *dst, int32_t N, int32_t C, int32_t H, int32_t W, int32_t cb,
+                               int32_t elem_size, unit_stream_t stream) {
+  return unit::nchwc<true>(src, dst, N, C, H, W, cb, elem_size, static_cast<hipStream_t>(stream), "unit_pack_nchwc");
+}
+
+extern "C" int unit_unpack_nchwc(const void *src, void *dst, int32_t N, int32_t C, int32_t H, int32_t W, int32_t cb,
+                                 int32_t elem_size, unit_stream_t stream) {
+  return unit::nchwc<false>(src, dst, N, C, H, W, cb, elem_size, static_cast<hipStream_t>(stream),
+                            "unit_unpack_nchwc");
+}
+
+extern "C" int unit_prepack_conv_weight_s8(const void *src, void *dst, int32_t O, int32_t I, int32_t KH, int32_t KW,
+                                           int32_t cb, unit_stream_t stream) {
+  using namespace unit;
+  const char *what = "unit_prepack_conv_weight_s8";
+  if (!src || !dst) return fail(UNIT_E_ARG, "%s: null pointer", what);
+  if (O <= 0 || I <= 0 || KH <= 0 || KW <= 0) return fail(UNIT_E_ARG, "%s: O, I, KH, KW must be positive", what);
+  if (cb != 16 && cb != 4) return fail(UNIT_E_ARG, "%s: cb must be 16 or 4 (got %d)", what, cb);
+  const int cc = ceil_div(I, cb), ko = ceil_div(O, 16);
+  const size_t words = (size_t)ko * cc * KH * KW * (cb / 4) * 16;
+  if (!fits(words * 4) || !fits((size_t)O * I * KH * KW)) return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
+  if (int rc = check_device()) return rc;
+  hipLaunchKernelGGL(prepack_conv_s8, dim3((unsigned)((words + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const signed char *>(src),
+                     static_cast<int *>(dst), O, I, KH, KW, cb, cc, words);
+  return launched(what);
+}
+
+extern "C" int unit_prepack_dense_weight_s8(const void *src, void *dst, int32_t N, int32_t K, unit_stream_t stream) {
+  using namespace unit;
+  const char *what = "unit_prepack_dense_weight_s8";
+  if (!src || !dst) return fail(UNIT_E_ARG, "%s: null pointer", what);
+  if (N <= 0 || K <= 0 || N % 128 || K % 4)
+    return fail(UNIT_E_ARG, "%s: N must be a positive multiple of 128 and K of 4 (got %d, %d)", what, N, K);
+  const size_t words = (size_t)N * K / 4;
+  if (!fits(words * 4)) return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
+  if (int rc = check_device()) return rc;
+  hipLaunchKernelGGL(prepack_dense_s8, dim3((unsigned)((words + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const int *>(src), static_cast<int *>(dst), K / 4,
+                     words);
+  return launched(what);
+}
+
+extern "C" int unit_prepack_conv_weight_f16(const void *src, void *dst, int32_t O, int32_t I, int32_t KH, int32_t KW,
+                                            unit_stream_t stream) {
+  using namespace unit;
+  const char *what = "unit_prepack_conv_weight_f16";
+  if (!src || !dst) return fail(UNIT_E_ARG, "%s: null pointer", what);
+  if (O <= 0 || I <= 0 || KH <= 0 || KW <= 0 || O % 16 || I % 16)
+    return fail(UNIT_E_ARG, "%s: O and I must be positive multiples of 16 (got %d, %d)", what, O, I);
+  const size_t total = (size_t)O * I * KH * KW;
+  if (!fits(total * 2)) return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
+  if (int rc = check_device()) return rc;
+  hipLaunchKernelGGL(prepack_conv_f16, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const unsigned short *>(src),
+                     static_cast<unsigned short *>(dst), I, KH, KW, total);
+  return launched(what);
+}

@@ -1,0 +1,214 @@
+// Tiled MFMA kernel shared by the int8 / fp16 GEMM and implicit-GEMM convolution entry points.
+//
+// One workgroup computes a BX x BY tile of  acc[x][y] = sum_k X[x][k] * Y[y][k]  where both
+// operand tiles are staged in LDS as rows of BKB reduction *bytes* (K-contiguous), 16-byte
+// chunks XOR-swizzled by row.  v_mfma_i32_32x32x32_i8 and v_mfma_f32_32x32x16_f16 both take
+// 32 reduction bytes per row per instruction (16 bytes per lane: lanes 0-31 the first chunk,
+// lanes 32-63 the second), so the byte-level tiling is identical for the two data types.
+//
+// X is the first MFMA operand (accumulator rows, spread over registers), Y the second
+// (accumulator columns, spread over lanes):  lane l, register r of a 32x32 block hold
+//   x = 8*(r/4) + 4*(l/32) + r%4,   y = l%32.
+//
+// Pipeline: global -> registers (one stage ahead) -> LDS (double buffered) -> MFMA, one
+// workgroup barrier per stage.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace unit {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef unsigned int u32;
+
+// 4-byte-aligned views for gathers whose address is only dword aligned
+typedef int v4i_a4 __attribute__((ext_vector_type(4), aligned(4)));
+
+struct OpI8 {
+  using acc_t = v16i;
+  using out_t = int;
+  using out4_t = v4i;
+  static constexpr bool kInt = true;
+  static __device__ __forceinline__ acc_t mma(v4i x, v4i y, acc_t c) {
+    return __builtin_amdgcn_mfma_i32_32x32x32_i8(x, y, c, 0, 0, 0);
+  }
+};
+
+struct OpF16 {
+  using acc_t = v16f;
+  using out_t = float;
+  using out4_t = v4f;
+  static constexpr bool kInt = false;
+  static __device__ __forceinline__ acc_t mma(v4i x, v4i y, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, x),
+                                                  __builtin_bit_cast(v8h, y), c, 0, 0, 0);
+  }
+};
+
+// XOR mask for the 16-byte chunk index of an LDS row.  Chosen so that any 8 (32 banks) or 16
+// (64 banks) consecutive rows reading the same logical chunk land on distinct banks, for rows
+// of 128 bytes (8 chunks) and of 64 bytes (4 chunks).
+template <int BKB>
+__device__ __forceinline__ int swz(int row) {
+  if constexpr (BKB == 128) {
+    return (row & 7) ^ ((row >> 3) & 1);
+  } else {
+    static_assert(BKB == 64, "LDS rows are 64 or 128 reduction bytes");
+    return ((row >> 1) & 3) ^ ((row >> 3) & 1);
+  }
+}
+
+template <int BKB>
+__device__ __forceinline__ int lds_off(int row, int chunk) {
+  return row * BKB + ((chunk ^ swz<BKB>(row)) << 4);
+}
+
+template <int BX_, int BY_, int BKB_, int WX_, int WY_>
+struct Tile {
+  static constexpr int BX = BX_, BY = BY_, BKB = BKB_, WX = WX_, WY = WY_;
+  static constexpr int NT = WX * WY * 64;
+  static constexpr int TX = BX / WX / 32, TY = BY / WY / 32;
+  static constexpr int CPR = BKB / 16;           // 16-byte chunks per LDS row
+  static constexpr int XBYTES = BX * BKB, YBYTES = BY * BKB;
+  static constexpr int STAGE = XBYTES + YBYTES;
+  static constexpr int LDS_TILES = 2 * STAGE;
+  static_assert(BX % (WX * 32) == 0 && BY % (WY * 32) == 0, "wave tile is a multiple of 32x32");
+};
+
+// Workgroup id -> tile coordinates.  Workgroups are dealt round-robin to the 8 XCDs, each with
+// its own L2: ids congruent mod 8 share an XCD, so they are given consecutive logical ids, and
+// logical ids walk the tile grid in panels `ph` X-tiles tall so that an XCD's working set is a
+// compact patch of the grid.
+struct GridMap {
+  int gx, gy, ph, total;
+  __device__ __forceinline__ void locate(int bid, int &bx, int &by) const {
+    constexpr int NXCD = 8;
+    int per = total / NXCD, rem = total % NXCD;
+    int xcd = bid % NXCD, idx = bid / NXCD;
+    int logical = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    int panel_sz = ph * gy;
+    int panel = logical / panel_sz, within = logical - panel * panel_sz;
+    int rows = gx - panel * ph;
+    rows = rows < ph ? rows : ph;
+    bx = panel * ph + within % rows;
+    by = within / rows;
+  }
+};
+
+enum { WS_NONE = 0, WS_X = 1, WS_Y = 2 };
+
+// The kernel.  XL / YL stage the operand tiles, Epi writes the accumulators.
+// WS selects which operand is the s8 weight whose per-row byte sums are accumulated on the side
+// (v_dot4 against 0x01010101): the u8 operand is staged as (u8 ^ 0x80) = u8 - 128 reinterpreted
+// as s8, because the MFMA int8 path multiplies signed by signed, and the epilogue adds back
+// 128 * sum_k w[k].
+template <class Op, class T, class XL, class YL, class Epi, int WS>
+__global__ __launch_bounds__(T::NT) void mma_kernel(typename XL::Params xp, typename YL::Params yp,
+                                                    typename Epi::Params ep, int nk, GridMap gm) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  const int t = threadIdx.x;
+  const int lane = t & 63, wave = t >> 6;
+  const int wx = wave % T::WX, wy = wave / T::WX;
+  const int l32 = lane & 31, half = lane >> 5;
+
+  int bx, by;
+  gm.locate(blockIdx.x, bx, by);
+  const int x0 = bx * T::BX, y0 = by * T::BY;
+
+  XL xl;
+  YL yl;
+  char *aux = lds + T::LDS_TILES;  // loader-private LDS (tap tables)
+  xl.init(xp, x0, t, aux);
+  yl.init(yp, y0, t, aux);
+
+  typename Op::acc_t acc[T::TX][T::TY];
+#pragma unroll
+  for (int i = 0; i < T::TX; ++i)
+#pragma unroll
+    for (int j = 0; j < T::TY; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+  int wsx[T::TX], wsy[T::TY];
+#pragma unroll
+  for (int i = 0; i < T::TX; ++i) wsx[i] = 0;
+#pragma unroll
+  for (int j = 0; j < T::TY; ++j) wsy[j] = 0;
+
+  // per-lane LDS read offsets (row part); the swizzle only depends on row % 16 and every
+  // 32-row block starts at a multiple of 32, so one mask serves all blocks of a lane
+  const int xrow = wx * (T::TX * 32) + l32, yrow = wy * (T::TY * 32) + l32;
+  const int xsw = swz<T::BKB>(xrow), ysw = swz<T::BKB>(yrow);
+
+  if (XL::kNeedsSync || YL::kNeedsSync) __syncthreads();  // tap tables visible
+  xl.fetch(0);
+  yl.fetch(0);
+  xl.commit(lds);
+  yl.commit(lds + T::XBYTES);
+  if (nk > 1) {
+    xl.fetch(1);
+    yl.fetch(1);
+  }
+  __syncthreads();
+
+  for (int kt = 0; kt < nk; ++kt) {
+    char *cur = lds + (kt & 1) * T::STAGE;
+    char *nxt = lds + ((kt & 1) ^ 1) * T::STAGE;
+    if (kt + 1 < nk) {  // registers hold stage kt+1
+      xl.commit(nxt);
+      yl.commit(nxt + T::XBYTES);
+    }
+    if (kt + 2 < nk) {
+      xl.fetch(kt + 2);
+      yl.fetch(kt + 2);
+    }
+    const char *xs = cur + xrow * T::BKB, *ys = cur + T::XBYTES + yrow * T::BKB;
+#pragma unroll
+    for (int kk = 0; kk < T::BKB / 32; ++kk) {
+      v4i xf[T::TX], yf[T::TY];
+#pragma unroll
+      for (int i = 0; i < T::TX; ++i)
+        xf[i] = *reinterpret_cast<const v4i *>(xs + i * 32 * T::BKB + (((2 * kk + half) ^ xsw) << 4));
+#pragma unroll
+      for (int j = 0; j < T::TY; ++j)
+        yf[j] = *reinterpret_cast<const v4i *>(ys + j * 32 * T::BKB + (((2 * kk + half) ^ ysw) << 4));
+      if constexpr (WS == WS_X) {
+#pragma unroll
+        for (int i = 0; i < T::TX; ++i)
+#pragma unroll
+          for (int d = 0; d < 4; ++d) wsx[i] = __builtin_amdgcn_sdot4(xf[i][d], 0x01010101, wsx[i], false);
+      }
+      if constexpr (WS == WS_Y) {
+#pragma unroll
+        for (int j = 0; j < T::TY; ++j)
+#pragma unroll
+          for (int d = 0; d < 4; ++d) wsy[j] = __builtin_amdgcn_sdot4(yf[j][d], 0x01010101, wsy[j], false);
+      }
+#pragma unroll
+      for (int i = 0; i < T::TX; ++i)
+#pragma unroll
+        for (int j = 0; j < T::TY; ++j) acc[i][j] = Op::mma(xf[i], yf[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+
+  // the two 32-lane halves hold the sums of the two 16-byte k-chunks of every MFMA step
+  if constexpr (WS == WS_X) {
+#pragma unroll
+    for (int i = 0; i < T::TX; ++i) wsx[i] += __shfl_xor(wsx[i], 32);
+  }
+  if constexpr (WS == WS_Y) {
+#pragma unroll
+    for (int j = 0; j < T::TY; ++j) wsy[j] += __shfl_xor(wsy[j], 32);
+  }
+
+  Epi::template store<T>(ep, acc, wsx, wsy, x0 + wx * (T::TX * 32), y0 + wy * (T::TY * 32), lane, wave,
+                         lds);
+}
+
+}  // namespace unit

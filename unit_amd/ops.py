@@ -1,0 +1,273 @@
+"""Operator entry points of the tensorized conv2d / dense / GEMM path, on torch tensors that live
+on the MI355X.  Same names, argument order and argument meaning as the reference operators they
+replace; every one hands raw device pointers to the C ABI in libunit_amd.so (hand-written gfx950
+kernels).  torch is used to allocate the result and to read shapes / pointers, nothing else.
+
+Reference call sites:
+  conv2d_NCHWc_int8        apps/cpu/kernel/conv2d.py:50-51   (topi.nn.conv2d_NCHWc_int8)
+  dense_dotprod            apps/cpu/kernel/int8-gemm.py:13-16 (topi.x86.dense_dotprod)
+  dense                    apps/cpu/relay/int8-gemm.py:14-16  (relay.nn.dense)
+  conv2d_NCHW16c_OHWI16o   python/tensorizer/ops/gpu.py:8-53  (_conv2d_NCHW16c_OHWI16o_impl)
+  gemm_fp16                apps/gpu/gemm.py:8-20
+"""
+import re
+
+import torch
+
+from . import _lib
+from ._lib import ConvDesc, check
+
+__all__ = [
+    "conv2d_NCHWc_int8", "dense_dotprod", "dense", "conv2d_NCHW16c_OHWI16o", "gemm_fp16",
+    "pack_nchwc", "unpack_nchwc", "prepack_conv_weight", "prepack_dense_weight",
+    "prepack_conv_weight_f16", "conv_out_hw", "last_variant",
+]
+
+
+# ------------------------------------------------------------------------------- helpers
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(t, name, dtype=None, ndim=None):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name}: expected a torch.Tensor, got {type(t).__name__}")
+    if not t.is_cuda:
+        raise ValueError(f"{name}: tensor must live on the GPU (there is no CPU implementation)")
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError(f"{name}: expected dtype {dtype}, got {t.dtype}")
+    if ndim is not None and t.dim() not in (ndim if isinstance(ndim, tuple) else (ndim,)):
+        raise ValueError(f"{name}: expected {ndim}-D tensor, got shape {tuple(t.shape)}")
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def _pair(v, name):
+    if isinstance(v, int):
+        return v, v
+    v = tuple(int(x) for x in v)
+    if len(v) != 2:
+        raise ValueError(f"{name}: expected an int or a pair, got {v}")
+    return v
+
+
+def _pad4(padding):
+    """TVM's get_pad_tuple: int -> all sides; (ph, pw) -> symmetric; (pt, pl, pb, pr)."""
+    if isinstance(padding, int):
+        return padding, padding, padding, padding
+    p = tuple(int(x) for x in padding)
+    if len(p) == 2:
+        return p[0], p[1], p[0], p[1]
+    if len(p) == 4:
+        return p
+    raise ValueError(f"padding: expected an int, (ph, pw) or (pt, pl, pb, pr), got {p}")
+
+
+def _layout_block(layout, name):
+    m = re.fullmatch(r"NCHW(\d+)c", layout)
+    if not m:
+        raise ValueError(f"{name}: expected a layout of the form NCHW<x>c, got {layout!r}")
+    return int(m.group(1))
+
+
+def conv_out_hw(h, w, kh, kw, stride, padding=0, dilation=1):
+    """Output height / width of a convolution, as the library computes it."""
+    sh, sw = _pair(stride, "stride")
+    dh, dw = _pair(dilation, "dilation")
+    pt, pl, pb, pr = _pad4(padding)
+    d = ConvDesc(1, 16, h, w, 16, kh, kw, sh, sw, pt, pl, pb, pr, dh, dw, 16)
+    import ctypes
+    oh, ow = ctypes.c_int32(), ctypes.c_int32()
+    check(_lib.load().unit_conv_out_hw(ctypes.byref(d), ctypes.byref(oh), ctypes.byref(ow)))
+    return oh.value, ow.value
+
+
+def last_variant():
+    """Kernel variant chosen by the last compute call (the analogue of the tuned-schedule index
+    the reference records per shape, python/tensorizer/tune.py:20-31)."""
+    return _lib.last_variant()
+
+
+# ------------------------------------------------------------------------------- int8
+def conv2d_NCHWc_int8(data, kernel, stride, padding, dilation=1, out_dtype="int32", layout="NCHW16c",
+                      out_layout="NCHW16c"):
+    """u8 x s8 -> i32 convolution on blocked layouts.
+
+    data   uint8 (N, C/cb, H, W, cb), cb in {16, 4}
+    kernel int8  (K/16, C/cb, KH, KW, cb/4, 16, 4)
+    returns int32 (N, K/16, OH, OW, 16)
+
+    As in TVM the channel block is taken from the tensor shapes; `layout` / `out_layout` are
+    checked for form only (the reference's driver passes 'NCHW4c' for 16-channel blocks too).
+    """
+    import ctypes
+    data = _dev(data, "data", torch.uint8, 5)
+    kernel = _dev(kernel, "kernel", torch.int8, 7)
+    if out_dtype != "int32":
+        raise ValueError(f"out_dtype: only 'int32' is supported, got {out_dtype!r}")
+    _layout_block(layout, "layout")
+    if _layout_block(out_layout, "out_layout") != 16:
+        raise ValueError("out_layout: the output channel block is 16 (NCHW16c)")
+    n, cc, h, w, cb = data.shape
+    ko, cc2, kh, kw, e, kb, i4 = kernel.shape
+    if cb not in (4, 16):
+        raise ValueError(f"data: channel block must be 16 or 4, got {cb}")
+    if (cc2, e, kb, i4) != (cc, cb // 4, 16, 4):
+        raise ValueError(f"kernel: shape {tuple(kernel.shape)} does not match data {tuple(data.shape)}; "
+                         f"expected (K/16, {cc}, KH, KW, {cb // 4}, 16, 4)")
+    sh, sw = _pair(stride, "stride")
+    dh, dw = _pair(dilation, "dilation")
+    pt, pl, pb, pr = _pad4(padding)
+    d = ConvDesc(n, cc * cb, h, w, ko * 16, kh, kw, sh, sw, pt, pl, pb, pr, dh, dw, cb)
+    L = _lib.load()
+    oh, ow = ctypes.c_int32(), ctypes.c_int32()
+    check(L.unit_conv_out_hw(ctypes.byref(d), ctypes.byref(oh), ctypes.byref(ow)))
+    out = torch.empty((n, ko, oh.value, ow.value, 16), dtype=torch.int32, device=data.device)
+    check(L.unit_conv2d_nchwc_u8s8s32(ctypes.byref(d), data.data_ptr(), kernel.data_ptr(), out.data_ptr(),
+                                      _stream()))
+    return out
+
+
+def dense_dotprod(data, weight, bias=None, out_dtype="int32"):
+    """u8 (M, K) x s8 packed (N/128, K/4, 128, 4) -> i32 (M, N) = data . W^T.
+    A 2-D weight (N, K) is taken as the un-packed relay.nn.dense operand."""
+    data = _dev(data, "data", torch.uint8, 2)
+    weight = _dev(weight, "weight", torch.int8, (2, 4))
+    if out_dtype != "int32":
+        raise ValueError(f"out_dtype: only 'int32' is supported, got {out_dtype!r}")
+    m, k = data.shape
+    L = _lib.load()
+    if weight.dim() == 4:
+        nb, kg, t, four = weight.shape
+        if (t, four) != (128, 4) or kg * 4 != k:
+            raise ValueError(f"weight: expected (N/128, {k // 4}, 128, 4), got {tuple(weight.shape)}")
+        n = nb * 128
+        out = torch.empty((m, n), dtype=torch.int32, device=data.device)
+        check(L.unit_dense_dotprod_u8s8s32(data.data_ptr(), weight.data_ptr(), out.data_ptr(), m, n, k, _stream()))
+    else:
+        n, k2 = weight.shape
+        if k2 != k:
+            raise ValueError(f"weight: expected (N, {k}), got {tuple(weight.shape)}")
+        out = torch.empty((m, n), dtype=torch.int32, device=data.device)
+        check(L.unit_dense_u8s8s32(data.data_ptr(), weight.data_ptr(), out.data_ptr(), m, n, k, _stream()))
+    if bias is not None:
+        out += _dev(bias, "bias", torch.int32)
+    return out
+
+
+def dense(data, weight, out_dtype="int32"):
+    """relay.nn.dense(x u8 (M, K), w s8 (N, K)) -> i32 (M, N)."""
+    weight = _dev(weight, "weight", torch.int8, 2)
+    return dense_dotprod(data, weight, None, out_dtype)
+
+
+# ------------------------------------------------------------------------------- fp16
+def gemm_fp16(a, b, out_dtype="float32"):
+    """c[x, y] = sum_k f32(a[x, k]) * f32(b[k, y]); a (M, K), b (K, N) fp16 row-major."""
+    a = _dev(a, "a", torch.float16, 2)
+    b = _dev(b, "b", torch.float16, 2)
+    if out_dtype not in ("float32", "float16"):
+        raise ValueError(f"out_dtype: expected 'float32' or 'float16', got {out_dtype!r}")
+    m, k = a.shape
+    k2, n = b.shape
+    if k2 != k:
+        raise ValueError(f"b: expected ({k}, N), got {tuple(b.shape)}")
+    half = out_dtype == "float16"
+    out = torch.empty((m, n), dtype=torch.float16 if half else torch.float32, device=a.device)
+    check(_lib.load().unit_gemm_f16(a.data_ptr(), b.data_ptr(), out.data_ptr(), m, n, k, int(half), _stream()))
+    return out
+
+
+def conv2d_NCHW16c_OHWI16o(a, b, stride_h, stride_w, out_type="float32"):
+    """fp16 valid convolution (no padding argument: callers pre-pad), fp32 accumulate.
+
+    Either a (N, C, H, W) + b (K, C, KH, KW), packed here exactly as the reference operator packs
+    them in-op, or a (N, C/16, H, W, 16) + b (K/16, C/16, KH, KW, 16 in, 16 out).
+    Returns float32 (N, K/16, OH, OW, 16)."""
+    import ctypes
+    if out_type != "float32":
+        raise ValueError(f"out_type: only 'float32' is supported, got {out_type!r}")
+    a = _dev(a, "a", torch.float16, (4, 5))
+    b = _dev(b, "b", torch.float16, (4, 6))
+    if a.dim() == 4 and b.dim() == 4:
+        if a.shape[1] % 16 or b.shape[0] % 16 or b.shape[1] != a.shape[1]:
+            raise ValueError("a, b: channel counts must match and be multiples of 16")
+        a = pack_nchwc(a, 16)
+        b = prepack_conv_weight_f16(b)
+    elif not (a.dim() == 5 and b.dim() == 6):
+        raise ValueError("a, b: expected 4-D + 4-D or 5-D + 6-D operands")
+    n, cc, h, w, cb = a.shape
+    ko, ib, kh, kw, ic, ob = b.shape
+    if cb != 16 or ic != 16 or ob != 16 or ib != cc:
+        raise ValueError(f"a {tuple(a.shape)} / b {tuple(b.shape)}: expected (N, C/16, H, W, 16) and "
+                         f"(K/16, C/16, KH, KW, 16, 16)")
+    d = ConvDesc(n, cc * 16, h, w, ko * 16, kh, kw, int(stride_h), int(stride_w), 0, 0, 0, 0, 1, 1, 16)
+    L = _lib.load()
+    oh, ow = ctypes.c_int32(), ctypes.c_int32()
+    check(L.unit_conv_out_hw(ctypes.byref(d), ctypes.byref(oh), ctypes.byref(ow)))
+    out = torch.empty((n, ko, oh.value, ow.value, 16), dtype=torch.float32, device=a.device)
+    check(L.unit_conv2d_nchw16c_f16f32(ctypes.byref(d), a.data_ptr(), b.data_ptr(), out.data_ptr(), _stream()))
+    return out
+
+
+# ------------------------------------------------------------------------------- layouts
+_ELEM = {torch.uint8: 1, torch.int8: 1, torch.float16: 2, torch.int32: 4, torch.float32: 4}
+
+
+def _elem(t, name):
+    if t.dtype not in _ELEM:
+        raise TypeError(f"{name}: unsupported dtype {t.dtype}")
+    return _ELEM[t.dtype]
+
+
+def pack_nchwc(x, cb):
+    """layout_transform NCHW -> NCHW{cb}c; channels are zero-padded up to a multiple of cb."""
+    x = _dev(x, "x", None, 4)
+    n, c, h, w = x.shape
+    out = torch.empty((n, -(-c // cb), h, w, cb), dtype=x.dtype, device=x.device)
+    check(_lib.load().unit_pack_nchwc(x.data_ptr(), out.data_ptr(), n, c, h, w, cb, _elem(x, "x"), _stream()))
+    return out
+
+
+def unpack_nchwc(x, channels=None):
+    """layout_transform NCHW{cb}c -> NCHW, keeping the first `channels` channels."""
+    x = _dev(x, "x", None, 5)
+    n, cc, h, w, cb = x.shape
+    c = cc * cb if channels is None else int(channels)
+    if not 0 < c <= cc * cb or -(-c // cb) != cc:
+        raise ValueError(f"channels: {c} does not fit {cc} blocks of {cb}")
+    out = torch.empty((n, c, h, w), dtype=x.dtype, device=x.device)
+    check(_lib.load().unit_unpack_nchwc(x.data_ptr(), out.data_ptr(), n, c, h, w, cb, _elem(x, "x"), _stream()))
+    return out
+
+
+def prepack_conv_weight(w, cb):
+    """int8 OIHW -> (ceil(O/16), ceil(I/cb), KH, KW, cb/4, 16, 4), zero-padded."""
+    w = _dev(w, "w", torch.int8, 4)
+    o, i, kh, kw = w.shape
+    if cb not in (4, 16):
+        raise ValueError(f"cb: must be 16 or 4, got {cb}")
+    out = torch.empty((-(-o // 16), -(-i // cb), kh, kw, cb // 4, 16, 4), dtype=torch.int8, device=w.device)
+    check(_lib.load().unit_prepack_conv_weight_s8(w.data_ptr(), out.data_ptr(), o, i, kh, kw, cb, _stream()))
+    return out
+
+
+def prepack_dense_weight(w):
+    """int8 (N, K) -> (N/128, K/4, 128, 4)."""
+    w = _dev(w, "w", torch.int8, 2)
+    n, k = w.shape
+    if n % 128 or k % 4:
+        raise ValueError(f"w: N must be a multiple of 128 and K of 4, got {tuple(w.shape)}")
+    out = torch.empty((n // 128, k // 4, 128, 4), dtype=torch.int8, device=w.device)
+    check(_lib.load().unit_prepack_dense_weight_s8(w.data_ptr(), out.data_ptr(), n, k, _stream()))
+    return out
+
+
+def prepack_conv_weight_f16(w):
+    """fp16 OIHW -> (O/16, I/16, KH, KW, 16 in, 16 out)."""
+    w = _dev(w, "w", torch.float16, 4)
+    o, i, kh, kw = w.shape
+    if o % 16 or i % 16:
+        raise ValueError(f"w: O and I must be multiples of 16, got {tuple(w.shape)}")
+    out = torch.empty((o // 16, i // 16, kh, kw, 16, 16), dtype=torch.float16, device=w.device)
+    check(_lib.load().unit_prepack_conv_weight_f16(w.data_ptr(), out.data_ptr(), o, i, kh, kw, _stream()))
+    return out
