@@ -1,0 +1,236 @@
+#!/usr/bin/env python3
+"""Benchmark of the tensorized conv2d / GEMM path on one MI355X.
+
+A step is one pass over the 53 convolutions of ResNet-50 v1 at batch 32 (20 unique layer shapes x
+their multiplicity), int8 u8 x s8 -> i32 in NCHW16c / NCHW4c, through the C ABI with operands and
+outputs already resident in HBM.  `value` is the whole-step throughput in TOP/s (2 x logical MACs /
+time).  The same line also carries the 4096^3 int8 and fp16 GEMMs, a per-layer table, the roofline
+of the layer that takes the largest share of the step, and the CPU baseline (the VNNI oracle on
+the host cores, same tensors, also used to check every GPU layer output bit for bit).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_INT8_TOPS = 5033.0   # MI355X dense int8 MFMA, published
+PEAK_F16_TFLOPS = 2516.0  # MI355X dense fp16 MFMA, published
+PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, published
+BATCH = 32
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / bit-exactness leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path is built and measured on ONE GPU; --gpus must be 1 "
+              "(nothing here shards across devices)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import unit_amd as U
+    from unit_amd import _lib, rng
+    from unit_amd import workloads as WL
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    L = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def dev_t(a):
+        return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+    def time_us(fn, iters, warm=3):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(iters):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        return s.elapsed_time(e) * 1e3 / iters
+
+    # ------------------------------------------------------------------ ResNet-50 b32 int8 conv stack
+    layers = []
+    for idx, s in enumerate(WL.RESNET50):
+        cb = WL.channel_block(s.C)
+        cp = -(-s.C // cb) * cb
+        data_np = rng.uniform_u8((BATCH, cp // cb, s.H, s.W, cb), 1000 + idx)
+        if cp != s.C:  # padded input channels hold zeros
+            data_np[..., s.C % cb:] = 0
+        w_oihw = rng.uniform_s8((s.K, s.C, s.KH, s.KW), 2000 + idx)
+        data = dev_t(data_np)
+        wt = U.prepack_conv_weight(dev_t(w_oihw), cb)
+        oh, ow = WL.out_hw(s)
+        out = torch.empty((BATCH, s.K // 16, oh, ow, 16), dtype=torch.int32, device=dev)
+        desc = _lib.ConvDesc(BATCH, cp, s.H, s.W, s.K, s.KH, s.KW, s.stride, s.stride, s.pad, s.pad, s.pad,
+                             s.pad, 1, 1, cb)
+        call = (lambda d=desc, x=data, w=wt, o=out: _lib.check(
+            L.unit_conv2d_nchwc_u8s8s32(ctypes.byref(d), x.data_ptr(), w.data_ptr(), o.data_ptr(), stream)))
+        call()
+        layers.append(dict(shape=s, cb=cb, data=data, data_np=data_np, wt=wt, out=out, call=call,
+                           variant=U.last_variant(), ops=2 * WL.macs(s, BATCH),
+                           bytes=WL.algorithmic_bytes(s, BATCH)))
+    torch.cuda.synchronize()
+
+    def step():
+        for ly in layers:
+            for _ in range(ly["shape"].count):
+                ly["call"]()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(args.steps):
+        step()
+    ev1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step = ev0.elapsed_time(ev1) / args.steps
+    step_ops = sum(ly["ops"] * ly["shape"].count for ly in layers)
+    value = step_ops / (ms_per_step * 1e-3) / 1e12
+
+    # per-layer launch duration (HIP events on the launch stream, back-to-back launches)
+    ridge = PEAK_INT8_TOPS * 1e12 / (PEAK_HBM_GBS * 1e9)
+    table = []
+    for ly in layers:
+        us = time_us(ly["call"], 30)
+        ai = ly["ops"] / ly["bytes"]
+        bound = "mfma" if ai >= ridge else "hbm"
+        tops, gbs = ly["ops"] / us / 1e6, ly["bytes"] / us / 1e3
+        frac = tops / PEAK_INT8_TOPS if bound == "mfma" else gbs / PEAK_HBM_GBS
+        ly["us"] = us
+        table.append(dict(layer=ly["shape"].name, count=ly["shape"].count, us=round(us, 2), tops=round(tops, 1),
+                          pct_int8_peak=round(100 * tops / PEAK_INT8_TOPS, 2), gbs=round(gbs, 1), bound=bound,
+                          frac=round(frac, 4), kernel=ly["variant"]))
+    dom = max(layers, key=lambda ly: ly["us"] * ly["shape"].count)
+    dom_row = table[layers.index(dom)]
+    if dom_row["bound"] == "mfma":
+        roofline = dict(bound="mfma", achieved=dom_row["tops"], peak=PEAK_INT8_TOPS, unit="TFLOP/s")
+    else:
+        roofline = dict(bound="hbm", achieved=dom_row["gbs"], peak=PEAK_HBM_GBS, unit="GB/s")
+    roofline.update(frac=dom_row["frac"], traffic=None, kernel=dom_row["kernel"], layer=dom_row["layer"],
+                    launch_us=dom_row["us"])
+
+    # ------------------------------------------------------------------ 4096^3 GEMMs
+    M = N = K = 4096
+    a8 = dev_t(rng.uniform_u8((M, K), 11))
+    w8_np = rng.uniform_s8((N, K), 12)
+    w8 = dev_t(w8_np)
+    wp8 = U.prepack_dense_weight(w8)
+    c8 = torch.empty((M, N), dtype=torch.int32, device=dev)
+    g_rm = lambda: _lib.check(L.unit_dense_u8s8s32(a8.data_ptr(), w8.data_ptr(), c8.data_ptr(), M, N, K, stream))
+    g_pk = lambda: _lib.check(L.unit_dense_dotprod_u8s8s32(a8.data_ptr(), wp8.data_ptr(), c8.data_ptr(), M, N, K,
+                                                            stream))
+    us_rm = time_us(g_rm, 30)
+    v_rm = U.last_variant()
+    us_pk = time_us(g_pk, 30)
+    v_pk = U.last_variant()
+    gemm_ops = 2.0 * M * N * K
+    gemm_i8 = dict(workload="int8 GEMM 4096^3 u8 x s8 -> i32",
+                   row_major=dict(us=round(us_rm, 2), tops=round(gemm_ops / us_rm / 1e6, 1),
+                                  pct_int8_peak=round(100 * gemm_ops / us_rm / 1e6 / PEAK_INT8_TOPS, 2), kernel=v_rm),
+                   vnni_packed=dict(us=round(us_pk, 2), tops=round(gemm_ops / us_pk / 1e6, 1),
+                                    pct_int8_peak=round(100 * gemm_ops / us_pk / 1e6 / PEAK_INT8_TOPS, 2),
+                                    kernel=v_pk))
+    ah_np = rng.normal_f16((M, K), 13, 1.0 / np.sqrt(K))
+    bh_np = rng.normal_f16((K, N), 14)
+    ah, bh = dev_t(ah_np), dev_t(bh_np)
+    cf = torch.empty((M, N), dtype=torch.float32, device=dev)
+    g_f = lambda: _lib.check(L.unit_gemm_f16(ah.data_ptr(), bh.data_ptr(), cf.data_ptr(), M, N, K, 0, stream))
+    us_f = time_us(g_f, 30)
+    v_f = U.last_variant()
+    # fp16 check on a 256 x 256 corner against float64
+    ref = ah_np[:256].astype(np.float64) @ bh_np[:, :256].astype(np.float64)
+    got = cf[:256, :256].cpu().numpy().astype(np.float64)
+    f16_err = float((np.abs(got - ref) / np.maximum(np.abs(ref), 1e-3 * np.abs(ref).max())).max())
+    gemm_f16 = dict(workload="fp16 GEMM 4096^3, fp32 accumulate, fp32 out", us=round(us_f, 2),
+                    tflops=round(gemm_ops / us_f / 1e6, 1),
+                    pct_f16_peak=round(100 * gemm_ops / us_f / 1e6 / PEAK_F16_TFLOPS, 2), kernel=v_f,
+                    max_rel_err=f16_err, tolerance=1e-2)
+
+    # ------------------------------------------------------------------ CPU baseline + bit-exactness
+    cpu_baseline = None
+    bit_exact = None
+    if not args.no_cpu:
+        from oracle import oracle as O  # the checker; also the timed CPU baseline ("port")
+        cores = len(os.sched_getaffinity(0))
+        cpu_s = 0.0
+        bit_exact = True
+        for ly in layers:
+            s = ly["shape"]
+            w_np = ly["wt"].cpu().numpy()
+            O.c_conv2d_nchwc(ly["data_np"][:1], w_np, s.stride, s.pad, 1)  # warm the thread pool
+            t1 = time.perf_counter()
+            ref = O.c_conv2d_nchwc(ly["data_np"], w_np, s.stride, s.pad, 1, impl="vnni", nthreads=cores)
+            cpu_s += (time.perf_counter() - t1) * s.count
+            ly["call"]()
+            torch.cuda.synchronize()
+            if not np.array_equal(ly["out"].cpu().numpy(), ref):
+                bit_exact = False
+                print(f"bench.py: MISMATCH vs oracle in layer {s.name}", file=sys.stderr)
+        g_rm()
+        torch.cuda.synchronize()
+        rows = 512
+        ref = O.c_dense(a8[:rows].cpu().numpy(), O.prepack_dense_weight(w8_np), nthreads=cores)
+        if not np.array_equal(c8[:rows].cpu().numpy(), ref):
+            bit_exact = False
+            print("bench.py: MISMATCH vs oracle in int8 GEMM", file=sys.stderr)
+        cpu_baseline = dict(value=round(step_ops / cpu_s / 1e12, 4), unit="TOP/s", cores=cores, kind="port",
+                            vnni=bool(O.has_vnni()),
+                            sample="one full pass of the same step (53 convolutions, batch 32) by the "
+                                   "AVX-512 VNNI oracle, each unique layer timed once x its multiplicity",
+                            seconds=round(cpu_s, 3))
+        gemm_i8["bit_exact_rows_checked"] = rows
+
+    line = {
+        "metric": "int8 conv2d TOPS & % int8 MFMA peak (ResNet-50 b32); fp16 GEMM TFLOPS",
+        "value": round(value, 2),
+        "unit": "TOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u8",
+        "data": "synthetic",
+        "config": {"workload": "ResNet-50 v1 conv stack (53 convolutions, 20 unique shapes), batch 32, int8 "
+                               "u8 x s8 -> i32, NCHW16c / NCHW4c stem (BASELINE configs[4])",
+                   "batch": BATCH, "ops_per_step": step_ops},
+        "pct_int8_mfma_peak": round(100 * value / PEAK_INT8_TOPS, 2),
+        "host_wall_ms_per_step": round(wall_ms, 4),
+        "bit_exact_vs_oracle": bit_exact,
+        "roofline": roofline,
+        "cpu_baseline": cpu_baseline,
+        "gemm_int8_4096": gemm_i8,
+        "gemm_fp16_4096": gemm_f16,
+        "layers": table,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

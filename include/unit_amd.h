@@ -144,6 +144,14 @@ int unit_prepack_conv_weight_f16(const void *src, void *dst, int32_t O, int32_t 
 int unit_mfma_tile_i8(const void *a, const void *b, void *c, unit_stream_t stream);
 int unit_mfma_tile_f16(const void *a, const void *b, void *c, unit_stream_t stream);
 
+/* Register-only MFMA throughput probe, the counterpart of the reference's vpdpbusd peak
+ * micro-benchmark (poc/vnni/micro.cc:16-51): `blocks` workgroups of 4 wavefronts each issue
+ * 4 * iters MFMAs per wavefront (int8 32x32x32 when f16 == 0, else fp16 32x32x16) on 4
+ * independent accumulator chains with no memory traffic.  Operations issued =
+ * blocks * 4 * 4 * iters * 65536 (int8) or * 32768 (fp16); the caller times the launch.
+ * `sink` is a 4-byte device scratch word. */
+int unit_mfma_peak(int32_t f16, int32_t blocks, int32_t iters, void *sink, unit_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -27,6 +27,7 @@ SYMBOLS = (
     "unit_prepack_conv_weight_f16",
     "unit_mfma_tile_i8",
     "unit_mfma_tile_f16",
+    "unit_mfma_peak",
 )
 
 
@@ -71,6 +72,7 @@ def load():
     L.unit_prepack_conv_weight_f16.argtypes = [vp, vp, i32, i32, i32, i32, vp]
     L.unit_mfma_tile_i8.argtypes = [vp, vp, vp, vp]
     L.unit_mfma_tile_f16.argtypes = [vp, vp, vp, vp]
+    L.unit_mfma_peak.argtypes = [i32, i32, i32, vp, vp]
     for name in SYMBOLS:
         fn = getattr(L, name)
         if name not in ("unit_last_error", "unit_last_variant"):

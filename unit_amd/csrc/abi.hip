@@ -1,5 +1,7 @@
 // C-ABI plumbing: version, thread-local error / variant strings, device check, convolution
 // geometry validation, and the single-instruction MFMA diagnostics.
+#include <stdlib.h>
+
 #include "host.hpp"
 #include "loaders.hpp"
 
@@ -13,6 +15,11 @@ char *error_buf() {
 char *variant_buf() {
   static thread_local char buf[96] = "";
   return buf;
+}
+
+int tuning_override(const char *name) {
+  const char *v = getenv(name);
+  return v ? atoi(v) : 0;
 }
 
 int check_device() {
@@ -100,8 +107,44 @@ __global__ __launch_bounds__(64) void mfma_tile_f16(const char *a, const char *b
   for (int r = 0; r < 16; ++r) c[(8 * (r >> 2) + 4 * half + (r & 3)) * 32 + l32] = acc[r];
 }
 
+// Register-only MFMA throughput probe in the manner of poc/vnni/micro.cc:16-51: 4 independent
+// accumulator chains per wave, no memory traffic; one workgroup of 4 waves per launch slot.
+template <class Op>
+__global__ __launch_bounds__(256) void mfma_peak(int iters, typename Op::out_t *sink) {
+  const int l = threadIdx.x;
+  v4i x = {l, l + 1, l + 2, l + 3}, y = {l ^ 5, l ^ 9, l ^ 3, l ^ 7};
+  if (!Op::kInt) {
+    x = v4i{0x3c003c00, 0x3c003c00, 0x3c003c00, 0x3c003c00};
+    y = x;
+  }
+  typename Op::acc_t a0, a1, a2, a3;
+  for (int r = 0; r < 16; ++r) a0[r] = a1[r] = a2[r] = a3[r] = 0;
+  for (int i = 0; i < iters; ++i) {
+    a0 = Op::mma(x, y, a0);
+    a1 = Op::mma(x, y, a1);
+    a2 = Op::mma(x, y, a2);
+    a3 = Op::mma(x, y, a3);
+  }
+  typename Op::out_t s = 0;
+  for (int r = 0; r < 16; ++r) s += a0[r] + a1[r] + a2[r] + a3[r];
+  if (s == (typename Op::out_t)12345) sink[0] = s;  // keeps the chains alive; practically never taken
+}
+
 }  // namespace
 }  // namespace unit
+
+extern "C" int unit_mfma_peak(int32_t f16, int32_t blocks, int32_t iters, void *sink, unit_stream_t stream) {
+  using namespace unit;
+  if (!sink || blocks <= 0 || iters <= 0) return fail(UNIT_E_ARG, "unit_mfma_peak: bad arguments");
+  if (int rc = check_device()) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (f16)
+    hipLaunchKernelGGL(mfma_peak<OpF16>, dim3(blocks), dim3(256), 0, s, iters, static_cast<float *>(sink));
+  else
+    hipLaunchKernelGGL(mfma_peak<OpI8>, dim3(blocks), dim3(256), 0, s, iters, static_cast<int *>(sink));
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "unit_mfma_peak: %s", hipGetErrorString(e));
+}
 
 extern "C" int unit_version(void) { return 100; }
 

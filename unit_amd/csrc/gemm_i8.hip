@@ -39,6 +39,15 @@ int dense(const void *a, const void *w, void *c, int M, int N, int K, unit_strea
   if (int rc = check_device()) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const long tiles_big = (long)ceil_div(M, 256) * ceil_div(N, 256);
+  switch (tuning_override("UNIT_AMD_DENSE_VARIANT")) {
+    case 1: return run_dense<Tile<256, 256, 128, 2, 2>, PACKED>(a, w, c, M, N, K, s);
+    case 2: return run_dense<Tile<256, 256, 64, 2, 4>, PACKED>(a, w, c, M, N, K, s);
+    case 3: return run_dense<Tile<256, 128, 64, 2, 2>, PACKED>(a, w, c, M, N, K, s);
+    case 4: return run_dense<Tile<128, 128, 64, 2, 2>, PACKED>(a, w, c, M, N, K, s);
+    case 5: return run_dense<Tile<256, 256, 64, 2, 2>, PACKED>(a, w, c, M, N, K, s);
+    case 6: return run_dense<Tile<128, 256, 128, 1, 4>, PACKED>(a, w, c, M, N, K, s);
+    default: break;
+  }
   if (M >= 256 && N >= 256 && tiles_big >= 128) return run_dense<Tile<256, 256, 128, 2, 4>, PACKED>(a, w, c, M, N, K, s);
   return run_dense<Tile<128, 128, 64, 2, 2>, PACKED>(a, w, c, M, N, K, s);
 }

@@ -29,6 +29,11 @@ inline void set_variant(const char *fmt, ...) {
   va_end(ap);
 }
 
+// Integer value of a tuning environment variable (0 when unset): lets a caller pin a kernel
+// variant per process, as the reference pins schedule indices through tensorizer.tune globals
+// (python/tensorizer/tune.py:3-16).
+int tuning_override(const char *name);
+
 int check_device();  // UNIT_OK or UNIT_E_DEVICE (message set)
 
 constexpr size_t kMaxTensorBytes = 0x7fffffffull;
