@@ -1,0 +1,81 @@
+"""The C-ABI library loads and exports every symbol include/unit_amd.h declares; argument
+validation that needs no GPU (nothing here launches a kernel)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_functions():
+    text = open(os.path.join(ROOT, "include", "unit_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(unit_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from unit_amd import _lib
+    lib = _lib.load()
+    names = header_functions()
+    assert len(names) >= 16
+    for n in names:
+        assert hasattr(lib, n), f"libunit_amd.so does not export {n}"
+    assert sorted(_lib.SYMBOLS) == names, "unit_amd/_lib.py and include/unit_amd.h disagree"
+    assert lib.unit_version() == 100
+
+
+def test_conv_desc_matches_the_header_struct():
+    from unit_amd import _lib
+    text = open(os.path.join(ROOT, "include", "unit_amd.h")).read()
+    body = re.search(r"typedef struct unit_conv_desc \{(.*?)\} unit_conv_desc;", text, flags=re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    fields = [f.strip() for decl in re.findall(r"int32_t ([^;]+);", body) for f in decl.split(",")]
+    assert fields == [f for f, _ in _lib.ConvDesc._fields_]
+    assert ctypes.sizeof(_lib.ConvDesc) == 4 * len(fields)
+
+
+def test_out_hw_and_error_paths_without_gpu():
+    from unit_amd import _lib
+    L = _lib.load()
+    oh, ow = ctypes.c_int32(), ctypes.c_int32()
+    d = _lib.ConvDesc(1, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 16)
+    assert L.unit_conv_out_hw(ctypes.byref(d), ctypes.byref(oh), ctypes.byref(ow)) == 0
+    assert (oh.value, ow.value) == (56, 56)
+    d = _lib.ConvDesc(1, 4, 224, 224, 64, 7, 7, 2, 2, 3, 3, 3, 3, 1, 1, 4)
+    assert L.unit_conv_out_hw(ctypes.byref(d), ctypes.byref(oh), ctypes.byref(ow)) == 0
+    assert (oh.value, ow.value) == (112, 112)
+    d = _lib.ConvDesc(1, 16, 4, 4, 16, 5, 5, 1, 1, 0, 0, 0, 0, 1, 1, 16)
+    assert L.unit_conv_out_hw(ctypes.byref(d), ctypes.byref(oh), ctypes.byref(ow)) == -1
+    assert b"window" in L.unit_last_error()
+    # null pointers and bad shapes are rejected before anything touches a device
+    assert L.unit_dense_u8s8s32(None, None, None, 4, 4, 16, None) == -1
+    assert L.unit_dense_dotprod_u8s8s32(1, 1, 1, 4, 100, 16, None) == -1 and b"multiple of 128" in L.unit_last_error()
+    assert L.unit_dense_u8s8s32(1, 1, 1, 4, 4, 10, None) == -1 and b"multiple of 16" in L.unit_last_error()
+    assert L.unit_gemm_f16(1, 1, 1, 4, 4, 5, 0, None) == -1
+    assert L.unit_pack_nchwc(1, 1, 1, 3, 4, 4, 4, 3, None) == -1 and b"elem_size" in L.unit_last_error()
+    assert L.unit_prepack_conv_weight_s8(1, 1, 16, 16, 3, 3, 8, None) == -1
+    bad = _lib.ConvDesc(1, 24, 8, 8, 16, 3, 3, 1, 1, 0, 0, 0, 0, 1, 1, 16)  # C % cb != 0
+    assert L.unit_conv2d_nchwc_u8s8s32(ctypes.byref(bad), 1, 1, 1, None) == -1
+    pad = _lib.ConvDesc(1, 16, 8, 8, 16, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 16)  # fp16 op has no padding argument
+    assert L.unit_conv2d_nchw16c_f16f32(ctypes.byref(pad), 1, 1, 1, None) == -1
+    with pytest.raises(ValueError):
+        _lib.check(-1)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from unit_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(_lib.UnitError, match="no CPU fallback"):
+        _lib.load()
+
+
+def test_product_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "unit_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".h")) or f == "Makefile":
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.lower(), f"{f} mentions the oracle"

@@ -92,3 +92,24 @@ def test_conv2d_fp16_unpacked_operands(dev, oracle):
     out = U.conv2d_NCHW16c_OHWI16o(_t(a, dev), _t(b, dev), 1, 1).cpu().numpy()
     ref = oracle.conv2d_nchw16c_f16(oracle.pack_nchwc(a, 16), oracle.prepack_conv_weight_f16(b), 1, 1)
     assert np.array_equal(out.astype(np.float64), ref)
+
+
+def test_fp16_golden_fixtures(dev):
+    import os
+    gold = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    g = np.load(os.path.join(gold, "fp16_gemm_24x36x40.npz"))
+    assert max_rel(U.gemm_fp16(_t(g["a"], dev), _t(g["b"], dev)).cpu().numpy(), g["out"]) <= REL_TOL
+    g = np.load(os.path.join(gold, "fp16_conv_3x3_c32_k32.npz"))
+    out = U.conv2d_NCHW16c_OHWI16o(_t(g["a"], dev), _t(g["b"], dev), 1, 1).cpu().numpy()
+    assert max_rel(out, g["out"]) <= REL_TOL
+
+
+def test_gemm_fp16_full_size(dev):
+    """4096^3: sampled rows against float64, tolerance 1e-2 max relative error."""
+    M = N = K = 4096
+    a = rng.normal_f16((M, K), 61, 1.0 / 64)
+    b = rng.normal_f16((K, N), 62)
+    out = U.gemm_fp16(_t(a, dev), _t(b, dev)).cpu().numpy()
+    rows = np.arange(0, M, 97)
+    ref = a[rows].astype(np.float64) @ b.astype(np.float64)
+    assert max_rel(out[rows], ref) <= REL_TOL

@@ -111,3 +111,50 @@ def test_conv2d_zero_padding_value(dev, oracle):
     out = U.conv2d_NCHWc_int8(_t(data, dev), _t(wt, dev), 1, 1).cpu().numpy()
     assert out[0, 0, 0, 0, 0] == 255 * 4 * C and out[0, 0, 2, 2, 0] == 255 * 9 * C
     assert np.array_equal(out, oracle.conv2d_nchwc_int8(data, wt, 1, 1))
+
+
+def _golden(pattern):
+    import glob
+    import os
+    return sorted(glob.glob(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", pattern)))
+
+
+@pytest.mark.parametrize("path", _golden("conv_*.npz"))
+def test_conv2d_golden_fixtures(dev, path):
+    g = np.load(path)
+    st, pad, dil, cb = (int(x) for x in g["params"])
+    out = U.conv2d_NCHWc_int8(_t(g["data"], dev), _t(g["weight"], dev), st, pad, dil, "int32", f"NCHW{cb}c")
+    assert np.array_equal(out.cpu().numpy(), g["out"])
+
+
+@pytest.mark.parametrize("path", _golden("dense_*.npz"))
+def test_dense_golden_fixtures(dev, path):
+    g = np.load(path)
+    assert np.array_equal(U.dense_dotprod(_t(g["a"], dev), _t(g["wp"], dev)).cpu().numpy(), g["out"])
+    assert np.array_equal(U.dense(_t(g["a"], dev), _t(g["w"], dev)).cpu().numpy(), g["out"])
+    assert np.array_equal(U.prepack_dense_weight(_t(g["w"], dev)).cpu().numpy(), g["wp"])
+
+
+def test_full_size_properties(dev):
+    """BASELINE-size checks that need no CPU reference: 4096^3 int8 GEMM and a batch-32 ResNet-50
+    layer through size-independent properties (linearity in the weights, the packed and un-packed
+    weight paths agree, all-ones weights give per-row activation sums)."""
+    M = N = K = 4096
+    a = _t(rng.uniform_u8((M, K), 41), dev)
+    w1 = rng.uniform_s8((N, K), 42) // 2
+    w2 = rng.uniform_s8((N, K), 43) // 2
+    c1 = U.dense(a, _t(w1.astype(np.int8), dev))
+    c2 = U.dense(a, _t(w2.astype(np.int8), dev))
+    c12 = U.dense(a, _t((w1 + w2).astype(np.int8), dev))
+    assert torch.equal(c12, c1 + c2)
+    assert torch.equal(U.dense_dotprod(a, U.prepack_dense_weight(_t(w1.astype(np.int8), dev))), c1)
+    ones = torch.ones((128, K), dtype=torch.int8, device=dev)
+    rowsum = a.to(torch.int32).sum(dim=1, dtype=torch.int32)
+    assert torch.equal(U.dense(a, ones), rowsum[:, None].expand(M, 128))
+    # batch-32 3x3 256 -> 256 @ 14: every image of a batch of identical images gives the same output,
+    # and equals the batch-1 result
+    d1 = rng.uniform_u8((1, 16, 14, 14, 16), 44)
+    wt = _t(rng.uniform_s8((16, 16, 3, 3, 4, 16, 4), 45), dev)
+    o1 = U.conv2d_NCHWc_int8(_t(d1, dev), wt, 1, 1)
+    o32 = U.conv2d_NCHWc_int8(_t(np.repeat(d1, 32, axis=0), dev), wt, 1, 1)
+    assert torch.equal(o32, o1.expand(32, -1, -1, -1, -1))
