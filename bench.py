@@ -33,6 +33,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / bit-exactness leg")
+    ap.add_argument("--no-graph", action="store_true", help="time eager launches only (no HIP graph replay)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus must be 1 "
@@ -84,7 +85,8 @@ def main():
         desc = _lib.ConvDesc(BATCH, cp, s.H, s.W, s.K, s.KH, s.KW, s.stride, s.stride, s.pad, s.pad, s.pad,
                              s.pad, 1, 1, cb)
         call = (lambda d=desc, x=data, w=wt, o=out: _lib.check(
-            L.unit_conv2d_nchwc_u8s8s32(ctypes.byref(d), x.data_ptr(), w.data_ptr(), o.data_ptr(), stream)))
+            L.unit_conv2d_nchwc_u8s8s32(ctypes.byref(d), x.data_ptr(), w.data_ptr(), o.data_ptr(),
+                                        torch.cuda.current_stream().cuda_stream)))
         call()
         layers.append(dict(shape=s, cb=cb, data=data, data_np=data_np, wt=wt, out=out, call=call,
                            variant=U.last_variant(), ops=2 * WL.macs(s, BATCH),
@@ -96,18 +98,44 @@ def main():
             for _ in range(ly["shape"].count):
                 ly["call"]()
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    ev0.record()
-    for _ in range(args.steps):
-        step()
-    ev1.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    ms_per_step = ev0.elapsed_time(ev1) / args.steps
+    def timed(run):
+        for _ in range(args.warmup):
+            run()
+        torch.cuda.synchronize()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        ev0.record()
+        for _ in range(args.steps):
+            run()
+        ev1.record()
+        torch.cuda.synchronize()
+        return ev0.elapsed_time(ev1) / args.steps, (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # eager: 53 C-ABI calls per step; graph: the same 53 launches captured once in a HIP graph
+    # and replayed (the library enqueues plain kernels only, so a step is capturable as is)
+    eager_ms, eager_wall_ms = timed(step)
+    launch_mode = "eager"
+    ms_per_step, wall_ms = eager_ms, eager_wall_ms
+    graph_ms = None
+    if not args.no_graph:
+        try:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                step()
+            graph_ms, graph_wall_ms = timed(graph.replay)
+            # replays must reproduce the eager outputs bit for bit
+            keep = [ly["out"].clone() for ly in layers]
+            for ly in layers:
+                ly["out"].fill_(-1)
+            graph.replay()
+            torch.cuda.synchronize()
+            same = all(torch.equal(k, ly["out"]) for k, ly in zip(keep, layers))
+            if same and graph_ms < eager_ms:
+                launch_mode, ms_per_step, wall_ms = "hipgraph", graph_ms, graph_wall_ms
+            elif not same:
+                print("bench.py: graph replay differs from eager launches; reporting eager", file=sys.stderr)
+        except Exception as ex:  # graph capture unavailable: the eager figure stands
+            print(f"bench.py: HIP graph capture failed ({ex}); reporting eager", file=sys.stderr)
     step_ops = sum(ly["ops"] * ly["shape"].count for ly in layers)
     value = step_ops / (ms_per_step * 1e-3) / 1e12
 
@@ -222,6 +250,9 @@ def main():
                    "batch": BATCH, "ops_per_step": step_ops},
         "pct_int8_mfma_peak": round(100 * value / PEAK_INT8_TOPS, 2),
         "host_wall_ms_per_step": round(wall_ms, 4),
+        "launch": launch_mode,
+        "eager_ms_per_step": round(eager_ms, 4),
+        "hipgraph_ms_per_step": None if graph_ms is None else round(graph_ms, 4),
         "bit_exact_vs_oracle": bit_exact,
         "roofline": roofline,
         "cpu_baseline": cpu_baseline,

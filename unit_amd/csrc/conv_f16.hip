@@ -27,7 +27,7 @@ int run_conv_f16(const unit_conv_desc *d, const ConvGeom &g0, const void *a, con
   typename Epi::Params ep{out, d->K, g.OH * g.OW, g.npix};
   const int gx = ceil_div(d->K, T::BX), gy = ceil_div(g.npix, T::BY);
   set_variant("f16conv_x%d_y%d_k%d_w%d", T::BX, T::BY, T::BKB, T::NT / 64);
-  return launch_mma<OpF16, T, XL, YL, Epi, WS_NONE>(xp, yp, ep, nk, gx, gy, gx, g.ntab * 8, s,
+  return launch_mma<OpF16, T, XL, YL, Epi, WS_NONE>(xp, yp, ep, nk, gx, gy, gx, 1, out, 0, g.ntab * 8, s,
                                                     "unit_conv2d_nchw16c_f16f32");
 }
 

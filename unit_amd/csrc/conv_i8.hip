@@ -1,55 +1,20 @@
-// int8 convolution in NCHW{16,4}c as an implicit GEMM: X operand = weights (rows = output
-// channels, read straight from the reference's (K/16, C/cb, KH, KW, cb/4, 16, 4) pre-pack),
-// Y operand = output pixels gathered on the fly from the u8 data tensor.
-#include "epilogues.hpp"
-#include "host.hpp"
-#include "loaders.hpp"
+// C-ABI entry of the int8 convolution: validates, plans (tile variant + k-splits) and dispatches.
+#include "conv_plan.hpp"
 
 namespace unit {
 
 int conv_geom(const unit_conv_desc *d, int tapb, ConvGeom *g, const char *what);  // abi.hip
+int conv_i8_c16(int variant, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w, void *out,
+                int splits, hipStream_t s);
+int conv_i8_c4(int variant, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w, void *out,
+               int splits, hipStream_t s);
 
 namespace {
-
-template <class T, int TAPB>
-int run_conv(const unit_conv_desc *d, const ConvGeom &g0, const void *data, const void *w, void *out,
-             hipStream_t s) {
-  using XL = VnniLoader<T::BX, T::BKB, T::NT, 16>;
-  using YL = ConvPixelLoader<T::BY, T::BKB, T::NT, TAPB, true>;
-  using Epi = ConvEpilogue<OpI8>;
-  ConvGeom g = g0;
-  const int kbytes = g.ntaps * TAPB;
-  const int nk = ceil_div(kbytes, T::BKB);
-  g.ntab = nk * T::BKB / TAPB;
-  typename XL::Params xp{static_cast<const char *>(w), d->K, kbytes / 4};
-  typename YL::Params yp{static_cast<const char *>(data), g};
-  typename Epi::Params ep{out, d->K, g.OH * g.OW, g.npix};
-  const int gx = ceil_div(d->K, T::BX), gy = ceil_div(g.npix, T::BY);
-  set_variant("i8conv_c%d_x%d_y%d_k%d_w%d", TAPB, T::BX, T::BY, T::BKB, T::NT / 64);
-  return launch_mma<OpI8, T, XL, YL, Epi, WS_X>(xp, yp, ep, nk, gx, gy, gx, g.ntab * 8, s,
-                                                "unit_conv2d_nchwc_u8s8s32");
-}
-
-template <int TAPB>
-int dispatch(const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w, void *out,
-             hipStream_t s) {
-  const int kbytes = g.ntaps * TAPB;
-  const bool k128 = kbytes % 128 == 0;
-  if (d->K % 256 == 0 && g.npix >= 256 * 64) {
-    if (k128) return run_conv<Tile<256, 256, 128, 2, 4>, TAPB>(d, g, data, w, out, s);
-    return run_conv<Tile<256, 256, 64, 2, 4>, TAPB>(d, g, data, w, out, s);
-  }
-  if (d->K % 128 == 0 && g.npix >= 256 * 32) {
-    if (k128) return run_conv<Tile<128, 256, 128, 2, 4>, TAPB>(d, g, data, w, out, s);
-    return run_conv<Tile<128, 256, 64, 2, 4>, TAPB>(d, g, data, w, out, s);
-  }
-  if (g.npix >= 256 * 32) {
-    if (k128) return run_conv<Tile<64, 256, 128, 1, 4>, TAPB>(d, g, data, w, out, s);
-    return run_conv<Tile<64, 256, 64, 1, 4>, TAPB>(d, g, data, w, out, s);
-  }
-  return run_conv<Tile<64, 64, 64, 2, 2>, TAPB>(d, g, data, w, out, s);
-}
-
+// measured on MI355X by `python -m unit_amd.tune` (key: N*OH*OW, K, C, KH, KW, stride)
+const TunedConv kTunedI8[] = {
+#include "tuned_conv_i8.inc"
+    {0, 0, 0, 0, 0, 0, 0, 0},
+};
 }  // namespace
 }  // namespace unit
 
@@ -64,5 +29,8 @@ extern "C" int unit_conv2d_nchwc_u8s8s32(const unit_conv_desc *d, const void *da
   if (!fits((size_t)g.npix * d->K * 4)) return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
   if (int rc = check_device()) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  return d->cb == 16 ? dispatch<16>(d, g, data, weight, out, s) : dispatch<4>(d, g, data, weight, out, s);
+  const int ntable = (int)(sizeof(kTunedI8) / sizeof(kTunedI8[0])) - 1;
+  const ConvPlan p = plan_conv(d, g.npix, g.ntaps * d->cb, kTunedI8, ntable, true);
+  return d->cb == 16 ? conv_i8_c16(p.variant, d, g, data, weight, out, p.splits, s)
+                     : conv_i8_c4(p.variant, d, g, data, weight, out, p.splits, s);
 }

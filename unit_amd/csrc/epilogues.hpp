@@ -14,9 +14,13 @@ struct GemmEpilogue {
     int M, N;
   };
   template <class T>
+  static constexpr int lds_bytes() {
+    return 0;
+  }
+  template <class T>
   static __device__ __forceinline__ void store(const Params &p, typename Op::acc_t (&acc)[T::TX][T::TY],
                                                int (&)[T::TX], int (&wsy)[T::TY], int xw0, int yw0, int lane,
-                                               int, char *) {
+                                               int, char *, bool accumulate) {
     const int l32 = lane & 31, half = lane >> 5;
 #pragma unroll
     for (int j = 0; j < T::TY; ++j) {
@@ -30,11 +34,18 @@ struct GemmEpilogue {
           if (m >= p.M) continue;
           const size_t idx = (size_t)m * p.N + n;
           if constexpr (Op::kInt) {
-            reinterpret_cast<int *>(p.c)[idx] = acc[i][j][r] + (wsy[j] << 7);
+            const int v = acc[i][j][r] + (wsy[j] << 7);
+            if (accumulate)
+              atomicAdd(reinterpret_cast<int *>(p.c) + idx, v);
+            else
+              reinterpret_cast<int *>(p.c)[idx] = v;
           } else if constexpr (OUT_F16) {
-            reinterpret_cast<_Float16 *>(p.c)[idx] = (_Float16)acc[i][j][r];
+            reinterpret_cast<_Float16 *>(p.c)[idx] = (_Float16)acc[i][j][r];  // no k-splits for f16 out
           } else {
-            reinterpret_cast<float *>(p.c)[idx] = acc[i][j][r];
+            if (accumulate)
+              unsafeAtomicAdd(reinterpret_cast<float *>(p.c) + idx, acc[i][j][r]);
+            else
+              reinterpret_cast<float *>(p.c)[idx] = acc[i][j][r];
           }
         }
     }
@@ -42,10 +53,14 @@ struct GemmEpilogue {
 };
 
 // Convolution output (N, K/16, OH, OW, 16), 4-byte elements: X rows are output channels, Y rows
-// are output pixels.  A lane holds one pixel and, per register quad, 4 consecutive channels ->
-// one 16-byte store; the two register quads q, q+1 of the two lane halves fill a pixel's
-// 64-byte channel block.  For int8 the weight is the X operand; its per-channel sums live in
-// other lanes, so they go through LDS once.
+// are output pixels.  In the accumulators a lane holds one pixel and, per register quad, 4
+// consecutive channels; written like that, a store instruction would scatter 16-byte pieces over
+// 32 pixels.  Each wave therefore transposes one 32 x 32 block at a time through its own LDS
+// scratch (32 pixels x 144-byte pitch, conflict-free 16-byte writes) and reads it back so that 64
+// lanes cover 16 pixels x 64 bytes = 1 KiB of consecutive output per store instruction.
+// LDS operations of one wave execute in order, so the scratch needs no barrier.
+// For int8 the weight is the X operand; its per-channel sums live in other lanes and go through
+// the same per-wave LDS area once.
 template <class Op>
 struct ConvEpilogue {
   struct Params {
@@ -54,40 +69,75 @@ struct ConvEpilogue {
     int ohw;   // OH * OW
     int npix;  // N * OH * OW
   };
+  static constexpr int kPitch = 144;               // bytes per pixel row of the scratch
+  static constexpr int kScratch = 32 * kPitch;     // per wave
+  // LDS bytes the epilogue needs for a tile shape
+  template <class T>
+  static constexpr int lds_bytes() {
+    return (T::NT / 64) * (kScratch + T::TX * 32 * 4);
+  }
+
   template <class T>
   static __device__ __forceinline__ void store(const Params &p, typename Op::acc_t (&acc)[T::TX][T::TY],
                                                int (&wsx)[T::TX], int (&)[T::TY], int xw0, int yw0, int lane,
-                                               int wave, char *lds) {
+                                               int wave, char *lds, bool accumulate) {
+    using out_t = typename Op::out_t;
+    using out4_t = typename Op::out4_t;
     const int l32 = lane & 31, half = lane >> 5;
-    int *wsb = reinterpret_cast<int *>(lds) + wave * (T::TX * 32);
+    char *scratch = lds + wave * kScratch;
+    int *wsb = reinterpret_cast<int *>(lds + (T::NT / 64) * kScratch) + wave * (T::TX * 32);
     if constexpr (Op::kInt) {
-      // the K loop ended with a workgroup barrier: the tile buffers are free
       if (half == 0) {
 #pragma unroll
         for (int i = 0; i < T::TX; ++i) wsb[i * 32 + l32] = wsx[i] << 7;
       }
-      __syncthreads();
     }
     const int ko_planes = p.K >> 4;
+    const int rp = lane >> 2, piece = lane & 3;  // read-back role: pixel row, 16-byte piece
 #pragma unroll
     for (int j = 0; j < T::TY; ++j) {
-      const int m = yw0 + j * 32 + l32;
-      if (m >= p.npix) continue;
-      const int n = m / p.ohw, pix = m - n * p.ohw;
-      typename Op::out_t *obase =
-          reinterpret_cast<typename Op::out_t *>(p.out) + ((size_t)n * ko_planes * p.ohw + pix) * 16;
+      // the two pixels this lane stores for block column j
+      size_t obase[2];
+      bool ok[2];
 #pragma unroll
-      for (int i = 0; i < T::TX; ++i)
+      for (int it = 0; it < 2; ++it) {
+        const int m = yw0 + j * 32 + it * 16 + rp;
+        ok[it] = m < p.npix;
+        const int n = m / p.ohw, pix = m - n * p.ohw;
+        obase[it] = ((size_t)n * ko_planes * p.ohw + pix) * 16 + piece * 4;
+      }
+#pragma unroll
+      for (int i = 0; i < T::TX; ++i) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int cl = i * 32 + 8 * q + 4 * half;  // channel inside the wave's X range
-          const int c = xw0 + cl;
-          if (c >= p.K) continue;
-          typename Op::out4_t v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
-                                   acc[i][j][4 * q + 3]};
+          out4_t v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
           if constexpr (Op::kInt) v += *reinterpret_cast<const v4i *>(wsb + cl);
-          *reinterpret_cast<typename Op::out4_t *>(obase + (size_t)(c >> 4) * p.ohw * 16 + (c & 15)) = v;
+          *reinterpret_cast<out4_t *>(scratch + l32 * kPitch + (8 * q + 4 * half) * 4) = v;
         }
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int c = xw0 + i * 32 + h * 16;  // first channel of this 16-channel plane
+          if (c >= p.K) continue;
+#pragma unroll
+          for (int it = 0; it < 2; ++it) {
+            const out4_t v = *reinterpret_cast<const out4_t *>(scratch + (it * 16 + rp) * kPitch + h * 64 + piece * 16);
+            if (!ok[it]) continue;
+            out_t *dst = reinterpret_cast<out_t *>(p.out) + obase[it] + (size_t)(c >> 4) * p.ohw * 16;
+            if (accumulate) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                if constexpr (Op::kInt)
+                  atomicAdd(dst + e, v[e]);
+                else
+                  unsafeAtomicAdd(dst + e, v[e]);
+              }
+            } else {
+              *reinterpret_cast<out4_t *>(dst) = v;
+            }
+          }
+        }
+      }
     }
   }
 };

@@ -17,7 +17,7 @@ int run_gemm_f16(const void *a, const void *b, void *c, int M, int N, int K, hip
   typename Epi::Params ep{c, M, N};
   const int nk = ceil_div(K * 2, T::BKB), gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
   set_variant("f16gemm_x%d_y%d_k%d_w%d%s", T::BX, T::BY, T::BKB, T::NT / 64, OUT_F16 ? "_h" : "");
-  return launch_mma<OpF16, T, XL, YL, Epi, WS_NONE>(xp, yp, ep, nk, gx, gy, 4, 0, s, "unit_gemm_f16");
+  return launch_mma<OpF16, T, XL, YL, Epi, WS_NONE>(xp, yp, ep, nk, gx, gy, 4, 1, c, 0, 0, s, "unit_gemm_f16");
 }
 
 template <bool OUT_F16>

@@ -3,6 +3,7 @@
 #include "epilogues.hpp"
 #include "host.hpp"
 #include "loaders.hpp"
+#include "mma_dma.hpp"
 
 namespace unit {
 namespace {
@@ -16,14 +17,47 @@ int run_dense(const void *a, const void *w, void *c, int M, int N, int K, hipStr
   typename XL::Params xp{static_cast<const char *>(a), M, K, K};
   typename Epi::Params ep{c, M, N};
   const int nk = ceil_div(K, T::BKB), gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
-  set_variant("i8dense%s_x%d_y%d_k%d_w%d", PACKED ? "pk" : "rm", T::BX, T::BY, T::BKB, T::NT / 64);
+  // few tiles and a long reduction: share K between workgroups (int32 atomics are exact)
+  int splits = tuning_override("UNIT_AMD_DENSE_SPLITK");
+  if (splits <= 0) {
+    splits = 1;  // atomics run at the memory side on this part: never faster in measurement
+  }
+  if (splits > nk) splits = nk;
+  if ((size_t)M * N * 4 % 16) splits = 1;
+  set_variant("i8dense%s_x%d_y%d_k%d_w%d_s%d", PACKED ? "pk" : "rm", T::BX, T::BY, T::BKB, T::NT / 64, splits);
   if constexpr (PACKED) {
     typename YLpk::Params yp{static_cast<const char *>(w), N, K / 4};
-    return launch_mma<OpI8, T, XL, YLpk, Epi, WS_Y>(xp, yp, ep, nk, gx, gy, 4, 0, s, "dense_dotprod");
+    return launch_mma<OpI8, T, XL, YLpk, Epi, WS_Y>(xp, yp, ep, nk, gx, gy, 4, splits, c, (size_t)M * N * 4, 0, s,
+                                                    "unit_dense_dotprod_u8s8s32");
   } else {
     typename YLrm::Params yp{static_cast<const char *>(w), N, K, K};
-    return launch_mma<OpI8, T, XL, YLrm, Epi, WS_Y>(xp, yp, ep, nk, gx, gy, 4, 0, s, "dense");
+    return launch_mma<OpI8, T, XL, YLrm, Epi, WS_Y>(xp, yp, ep, nk, gx, gy, 4, splits, c, (size_t)M * N * 4, 0, s,
+                                                    "unit_dense_u8s8s32");
   }
+}
+
+// direct-to-LDS variant: row-major weights, K a whole number of stages
+template <class T, int NSTAGE>
+int run_dense_dma(const void *a, const void *w, void *c, int M, int N, int K, hipStream_t s) {
+  using Epi = GemmEpilogue<OpI8, false>;
+  DmaParams p{static_cast<const char *>(a), static_cast<const char *>(w), M, N, K};
+  typename Epi::Params ep{c, M, N};
+  const int nk = K / T::BKB, gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
+  constexpr int lds = NSTAGE * T::STAGE;
+  static_assert(lds <= kMaxLds, "ring does not fit the LDS");
+  auto kern = mma_dma_kernel<OpI8, T, NSTAGE, Epi, WS_Y, true>;
+  static thread_local bool allowed = false;
+  if (!allowed) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
+    if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "unit_dense_u8s8s32: hipFuncSetAttribute: %s", hipGetErrorString(e));
+    allowed = true;
+  }
+  GridMap gm{gx, gy, gx < 4 ? gx : 4, 1, gx * gy};
+  set_variant("i8densedma_x%d_y%d_k%d_w%d_r%d", T::BX, T::BY, T::BKB, T::NT / 64, NSTAGE);
+  hipLaunchKernelGGL(kern, dim3(gm.total), dim3(T::NT), lds, s, p, ep, nk, gm);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "unit_dense_u8s8s32: launch: %s", hipGetErrorString(e));
 }
 
 template <bool PACKED>
@@ -46,6 +80,12 @@ int dense(const void *a, const void *w, void *c, int M, int N, int K, unit_strea
     case 4: return run_dense<Tile<128, 128, 64, 2, 2>, PACKED>(a, w, c, M, N, K, s);
     case 5: return run_dense<Tile<256, 256, 64, 2, 2>, PACKED>(a, w, c, M, N, K, s);
     case 6: return run_dense<Tile<128, 256, 128, 1, 4>, PACKED>(a, w, c, M, N, K, s);
+    case 7: if (!PACKED && K % 64 == 0) return run_dense_dma<Tile<256, 256, 64, 2, 2>, 4>(a, w, c, M, N, K, s); break;
+    case 8: if (!PACKED && K % 64 == 0) return run_dense_dma<Tile<256, 256, 64, 2, 4>, 4>(a, w, c, M, N, K, s); break;
+    case 9: if (!PACKED && K % 128 == 0) return run_dense_dma<Tile<256, 256, 128, 2, 2>, 2>(a, w, c, M, N, K, s); break;
+    case 10: if (!PACKED && K % 64 == 0) return run_dense_dma<Tile<256, 256, 64, 2, 2>, 3>(a, w, c, M, N, K, s); break;
+    case 11: if (!PACKED && K % 64 == 0) return run_dense_dma<Tile<256, 128, 64, 2, 2>, 4>(a, w, c, M, N, K, s); break;
+    case 12: if (!PACKED && K % 128 == 0) return run_dense_dma<Tile<256, 256, 128, 2, 4>, 2>(a, w, c, M, N, K, s); break;
     default: break;
   }
   if (M >= 256 && N >= 256 && tiles_big >= 128) return run_dense<Tile<256, 256, 128, 2, 4>, PACKED>(a, w, c, M, N, K, s);

@@ -43,22 +43,39 @@ inline bool fits(size_t bytes) { return bytes <= kMaxTensorBytes; }
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
+// Enqueue mma_kernel over gx x gy tiles and `splits` k-ranges.  With splits > 1 the epilogue
+// accumulates with atomics, so `out` (out_bytes, a multiple of 16) is zero-filled first.
 template <class Op, class T, class XL, class YL, class Epi, int WS>
 int launch_mma(const typename XL::Params &xp, const typename YL::Params &yp, const typename Epi::Params &ep,
-               int nk, int gx, int gy, int ph, int aux_bytes, hipStream_t stream, const char *what) {
-  const int lds = T::LDS_TILES + aux_bytes;
+               int nk, int gx, int gy, int ph, int splits, void *out, size_t out_bytes, int aux_bytes,
+               hipStream_t stream, const char *what) {
+  constexpr int epi = Epi::template lds_bytes<T>();
+  const int lds = (T::LDS_TILES + aux_bytes) > epi ? (T::LDS_TILES + aux_bytes) : epi;
   if (lds > kMaxLds) return fail(UNIT_E_ARG, "%s: needs %d bytes of LDS (limit %d)", what, lds, kMaxLds);
   auto kern = mma_kernel<Op, T, XL, YL, Epi, WS>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-  if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "%s: hipFuncSetAttribute: %s", what, hipGetErrorString(e));
+  // the opt-in for > 64 KiB of dynamic LDS is sticky per kernel; raise it only when needed
+  static thread_local int lds_allowed = 0;
+  if (lds > lds_allowed) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
+    if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "%s: hipFuncSetAttribute: %s", what, hipGetErrorString(e));
+    lds_allowed = kMaxLds;
+  }
+  if (splits < 1) splits = 1;
+  if (splits > nk) splits = nk;
+  if (splits > 1) {
+    const size_t n16 = out_bytes / 16;
+    hipLaunchKernelGGL(zero_fill, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, stream,
+                       static_cast<v4i *>(out), n16);
+  }
   GridMap gm;
   gm.gx = gx;
   gm.gy = gy;
   gm.ph = ph < 1 ? 1 : (ph > gx ? gx : ph);
-  gm.total = gx * gy;
+  gm.splits = splits;
+  gm.total = gx * gy * splits;
   hipLaunchKernelGGL(kern, dim3(gm.total), dim3(T::NT), lds, stream, xp, yp, ep, nk, gm);
-  e = hipGetLastError();
+  hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "%s: launch: %s", what, hipGetErrorString(e));
   return UNIT_OK;
 }

@@ -12,7 +12,7 @@ __device__ __forceinline__ v4i zero4() { return v4i{0, 0, 0, 0}; }
 // Thread t owns chunk column t % CPR of rows t / CPR + i * NT / CPR: 8 (or 4) consecutive lanes
 // read one whole 128-byte (64-byte) row segment.
 // ------------------------------------------------------------------------------------------
-template <int ROWS, int BKB, int NT, bool XOR80>
+template <int ROWS, int BKB, int NT, bool XOR80, int PF = 1>
 struct RowMajorLoader {
   struct Params {
     const char *base;
@@ -21,18 +21,22 @@ struct RowMajorLoader {
     int kbytes;  // valid reduction bytes per row (multiple of 16)
   };
   static constexpr bool kNeedsSync = false;
+  static constexpr int kPF = PF;
   static constexpr int CPR = BKB / 16, RPP = NT / CPR, NCH = ROWS / RPP;
   static_assert(NT % CPR == 0 && ROWS % RPP == 0 && RPP % 16 == 0, "row-major loader shape");
 
-  v4i r[NCH];
+  v4i r[PF][NCH];
   u32 off[NCH];
+  bool okm[PF];  // stage in the slot lies inside the reduction (else it is staged as zeros)
   const char *base;
+  int coff;    // byte offset of the thread's chunk column inside a stage
   int kleft;   // kbytes - c*16: chunk of stage kt is valid iff kt*BKB < kleft
   int ldsoff;  // LDS offset of chunk 0
 
   __device__ __forceinline__ void init(const Params &p, int row0, int t, char *) {
     const int c = t % CPR, rr = t / CPR;
-    base = p.base + c * 16;
+    base = p.base;
+    coff = c * 16;
     kleft = p.kbytes - c * 16;
     ldsoff = lds_off<BKB>(rr, c);
 #pragma unroll
@@ -42,17 +46,21 @@ struct RowMajorLoader {
       off[i] = (u32)row * (u32)p.ld;
     }
   }
+  template <int S>
   __device__ __forceinline__ void fetch(int kt) {
-    const int kb = kt * BKB;
-    const bool ok = kb < kleft;
+    // loads are unconditional (no branches in the pipeline): a chunk past the end of the
+    // reduction re-reads the first chunk of the row and is zeroed when it is written to LDS
+    const bool ok = kt * BKB < kleft;
+    const int kb = ok ? kt * BKB + coff : 0;
+    okm[S] = ok;
 #pragma unroll
-    for (int i = 0; i < NCH; ++i)
-      r[i] = ok ? *reinterpret_cast<const v4i *>(base + off[i] + kb) : zero4();
+    for (int i = 0; i < NCH; ++i) r[S][i] = *reinterpret_cast<const v4i *>(base + off[i] + kb);
   }
+  template <int S>
   __device__ __forceinline__ void commit(char *tile) {
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      v4i v = r[i];
+      v4i v = okm[S] ? r[S][i] : zero4();
       if (XOR80) v ^= (int)0x80808080;
       *reinterpret_cast<v4i *>(tile + ldsoff + i * RPP * BKB) = v;
     }
@@ -66,7 +74,7 @@ struct RowMajorLoader {
 // A thread loads, for 4 consecutive n, the 4 k-groups of one 16-byte reduction chunk (4 x 16
 // bytes), transposes the 4x4 dwords in registers (free) and writes one 16-byte LDS chunk per n.
 // ------------------------------------------------------------------------------------------
-template <int ROWS, int BKB, int NT, int NB>
+template <int ROWS, int BKB, int NT, int NB, int PF = 1>
 struct VnniLoader {
   struct Params {
     const char *base;
@@ -74,17 +82,19 @@ struct VnniLoader {
     int kg_total;  // k-groups per n
   };
   static constexpr bool kNeedsSync = false;
+  static constexpr int kPF = PF;
   static constexpr int CPR = BKB / 16, QUADS = ROWS / 4, UNITS = QUADS * CPR;
   static constexpr int UPT = (UNITS + NT - 1) / NT;
   static constexpr bool kAllActive = UNITS % NT == 0;  // else UNITS < NT: threads >= UNITS idle
   static_assert(kAllActive || UNITS < NT, "vnni loader shape");
 
-  v4i r[UPT][4];
-  const char *ptr[UPT];  // address of k-group 4*c of the thread's 4 n
+  v4i r[PF][UPT][4];
+  const char *ptr[UPT];  // address of k-group 0 of the thread's 4 n
   int cidx[UPT];         // chunk column inside the stage
   int lrow[UPT];         // first LDS row (n quad)
   int kg_total;
   int kgstride;          // bytes between consecutive k-groups
+  int kt_of[PF];         // stage held by each slot (its k-groups are re-checked at commit)
   bool active;
 
   __device__ __forceinline__ void init(const Params &p, int row0, int t, char *) {
@@ -93,34 +103,42 @@ struct VnniLoader {
     active = kAllActive || t < UNITS;
 #pragma unroll
     for (int i = 0; i < UPT; ++i) {
-      const int u = i * NT + t;
+      const int u = (i * NT + t) % UNITS;  // idle threads shadow a live unit (their loads stay in bounds)
       const int nq = u % QUADS, c = u / QUADS;
       int n = row0 + nq * 4;
       n = n < p.rows ? n : p.rows - 4;
       cidx[i] = c;
       lrow[i] = nq * 4;
-      ptr[i] = p.base + ((size_t)(n / NB) * p.kg_total) * (NB * 4) + (n % NB) * 4 + (size_t)(4 * c) * (NB * 4);
+      ptr[i] = p.base + ((size_t)(n / NB) * p.kg_total) * (NB * 4) + (n % NB) * 4;
     }
   }
+  template <int S>
   __device__ __forceinline__ void fetch(int kt) {
+    kt_of[S] = kt;
 #pragma unroll
     for (int i = 0; i < UPT; ++i) {
       const int kg0 = (kt * CPR + cidx[i]) * 4;
-      const char *q = ptr[i] + (size_t)(kt * CPR * 4) * kgstride;
 #pragma unroll
-      for (int d = 0; d < 4; ++d)
-        r[i][d] = (active && kg0 + d < kg_total) ? *reinterpret_cast<const v4i *>(q + d * kgstride) : zero4();
+      for (int d = 0; d < 4; ++d) {
+        // unconditional load: a k-group past the end re-reads k-group 0
+        const int kg = kg0 + d < kg_total ? kg0 + d : 0;
+        r[S][i][d] = *reinterpret_cast<const v4i *>(ptr[i] + (size_t)kg * kgstride);
+      }
     }
   }
+  template <int S>
   __device__ __forceinline__ void commit(char *tile) {
     if (!active) return;
 #pragma unroll
-    for (int i = 0; i < UPT; ++i)
+    for (int i = 0; i < UPT; ++i) {
+      const int left = kg_total - (kt_of[S] * CPR + cidx[i]) * 4;  // valid k-groups of this chunk
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        v4i v = {r[i][0][j], r[i][1][j], r[i][2][j], r[i][3][j]};
+        v4i v = {left > 0 ? r[S][i][0][j] : 0, left > 1 ? r[S][i][1][j] : 0, left > 2 ? r[S][i][2][j] : 0,
+                 left > 3 ? r[S][i][3][j] : 0};
         *reinterpret_cast<v4i *>(tile + lds_off<BKB>(lrow[i] + j, cidx[i])) = v;
       }
+    }
   }
 };
 
@@ -130,7 +148,7 @@ struct VnniLoader {
 // + (n % NBLK) * 2.  A thread loads an 8 (k) x 4 (n) patch as 8 x 8 bytes, transposes it with
 // v_perm_b32 and writes one 16-byte chunk (8 k) per n.
 // ------------------------------------------------------------------------------------------
-template <int ROWS, int BKB, int NT>
+template <int ROWS, int BKB, int NT, int PF = 1>
 struct KMajorF16Loader {
   struct Params {
     const char *base;
@@ -141,15 +159,17 @@ struct KMajorF16Loader {
     int row_stride;    // bytes between consecutive k
   };
   static constexpr bool kNeedsSync = false;
+  static constexpr int kPF = PF;
   static constexpr int CPR = BKB / 16, QUADS = ROWS / 4, UNITS = QUADS * CPR;
   static constexpr int UPT = (UNITS + NT - 1) / NT;
   static constexpr bool kAllActive = UNITS % NT == 0;  // else UNITS < NT: threads >= UNITS idle
   static_assert(kAllActive || UNITS < NT, "k-major loader shape");
 
-  v2i r[UPT][8];
+  v2i r[PF][UPT][8];
   const char *ptr[UPT];
   int cidx[UPT], lrow[UPT];
   int ktotal, row_stride;
+  bool okm[PF][UPT];
   bool active;
 
   __device__ __forceinline__ void init(const Params &p, int row0, int t, char *) {
@@ -158,27 +178,29 @@ struct KMajorF16Loader {
     active = kAllActive || t < UNITS;
 #pragma unroll
     for (int i = 0; i < UPT; ++i) {
-      const int u = i * NT + t;
+      const int u = (i * NT + t) % UNITS;  // idle threads shadow a live unit
       const int nq = u % QUADS, c = u / QUADS;
       int n = row0 + nq * 4;
       n = n < p.rows ? n : p.rows - 4;
       cidx[i] = c;
       lrow[i] = nq * 4;
-      ptr[i] = p.base + (size_t)(n / p.nblk) * p.blk_stride + (size_t)(n % p.nblk) * 2 +
-               (size_t)(8 * c) * p.row_stride;
+      ptr[i] = p.base + (size_t)(n / p.nblk) * p.blk_stride + (size_t)(n % p.nblk) * 2;
     }
   }
+  template <int S>
   __device__ __forceinline__ void fetch(int kt) {
 #pragma unroll
     for (int i = 0; i < UPT; ++i) {
       const int k0 = (kt * CPR + cidx[i]) * 8;
-      const char *q = ptr[i] + (size_t)(kt * CPR * 8) * row_stride;
-      const bool ok = active && k0 < ktotal;  // ktotal % 8 == 0: a chunk is all valid or all padding
+      const bool ok = k0 < ktotal;  // ktotal % 8 == 0: a chunk is all valid or all padding
+      // unconditional loads: a chunk past the end re-reads rows 0..7
+      const char *q = ptr[i] + (ok ? (size_t)k0 * row_stride : 0);
+      okm[S][i] = ok;
 #pragma unroll
-      for (int kk = 0; kk < 8; ++kk)
-        r[i][kk] = ok ? *reinterpret_cast<const v2i *>(q + (size_t)kk * row_stride) : v2i{0, 0};
+      for (int kk = 0; kk < 8; ++kk) r[S][i][kk] = *reinterpret_cast<const v2i *>(q + (size_t)kk * row_stride);
     }
   }
+  template <int S>
   __device__ __forceinline__ void commit(char *tile) {
     if (!active) return;
 #pragma unroll
@@ -190,7 +212,7 @@ struct KMajorF16Loader {
         v4i v;
 #pragma unroll
         for (int p = 0; p < 4; ++p)
-          v[p] = (int)__builtin_amdgcn_perm((u32)r[i][2 * p + 1][j >> 1], (u32)r[i][2 * p][j >> 1], sel);
+          v[p] = okm[S][i] ? (int)__builtin_amdgcn_perm((u32)r[S][i][2 * p + 1][j >> 1], (u32)r[S][i][2 * p][j >> 1], sel) : 0;
         *reinterpret_cast<v4i *>(tile + lds_off<BKB>(lrow[i] + j, cidx[i])) = v;
       }
   }
@@ -217,21 +239,23 @@ struct ConvGeom {
   u32 img_bytes;  // bytes per image
 };
 
-template <int ROWS, int BKB, int NT, int TAPB, bool XOR80>
+template <int ROWS, int BKB, int NT, int TAPB, bool XOR80, int PF = 1>
 struct ConvPixelLoader {
   struct Params {
     const char *base;
     ConvGeom g;
   };
   static constexpr bool kNeedsSync = true;
+  static constexpr int kPF = PF;
   static constexpr int CPR = BKB / 16;
   static constexpr int PPT = ROWS > NT ? ROWS / NT : 1;   // pixels per thread
   static constexpr int TPS = NT > ROWS ? NT / ROWS : 1;   // threads sharing a pixel
   static constexpr int NCH = ROWS * CPR / NT;
   static constexpr int CPT = NCH / PPT;                   // chunk columns per thread
-  static_assert((ROWS % NT == 0 || NT % ROWS == 0) && NCH >= 1 && CPR % TPS == 0, "pixel loader shape");
+  static_assert((ROWS % NT == 0 || NT % ROWS == 0) && NCH >= 1 && NCH <= 8 && CPR % TPS == 0, "pixel loader shape");
 
-  v4i r[NCH];
+  v4i r[PF][NCH];
+  u32 okm[PF];      // bit (4*i + d): dword d of chunk i comes from inside the image
   int pixoff[PPT];  // byte offset of (n, oh*sh-pt, ow*sw-pl) in the data tensor; INT_MIN/2 = no pixel
   int ih0[PPT], iw0[PPT];
   const char *base;
@@ -276,38 +300,56 @@ struct ConvPixelLoader {
     }
   }
 
-  __device__ __forceinline__ bool tap_addr(int tap, int s, const char *&src) const {
-    const v2i e = tab[tap];
+  // address of a tap's input pixel, or of the tensor start when the tap falls outside the image
+  // (zero padding, no pixel, past the last tap): loads stay unconditional and in bounds
+  __device__ __forceinline__ bool tap_addr(v2i e, int s, const char *&src) const {
     const int ih = ih0[s] + (e[1] & 0xffff), iw = iw0[s] + (e[1] >> 16);
-    src = base + pixoff[s] + e[0];
-    return (u32)ih < (u32)H && (u32)iw < (u32)W;
+    const bool ok = (u32)ih < (u32)H && (u32)iw < (u32)W;
+    src = base + (ok ? pixoff[s] + e[0] : 0);
+    return ok;
   }
 
+  template <int S>
   __device__ __forceinline__ void fetch(int kt) {
+    constexpr int TPC = TAPB == 4 ? 4 : 1;  // table entries per chunk
+    v2i ent[NCH][TPC];
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int g = kt * CPR + (i / PPT) * TPS + tq;  // global chunk index
+#pragma unroll
+      for (int d = 0; d < TPC; ++d) ent[i][d] = tab[TAPB == 4 ? 4 * g + d : (TAPB == 32 ? g >> 1 : g)];
+    }
+    u32 m = 0;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       const int s = i % PPT;
-      const int g = kt * CPR + (i / PPT) * TPS + tq;  // global chunk index
+      const int g = kt * CPR + (i / PPT) * TPS + tq;
       const char *src;
-      if constexpr (TAPB == 16) {
-        r[i] = tap_addr(g, s, src) ? *reinterpret_cast<const v4i *>(src) : zero4();
-      } else if constexpr (TAPB == 32) {
-        const bool ok = tap_addr(g >> 1, s, src);
-        r[i] = ok ? *reinterpret_cast<const v4i *>(src + (g & 1) * 16) : zero4();
-      } else {
-        static_assert(TAPB == 4 || TAPB == 16 || TAPB == 32, "tap width");
+      if constexpr (TAPB == 4) {
         v4i v;
 #pragma unroll
-        for (int d = 0; d < 4; ++d) v[d] = tap_addr(4 * g + d, s, src) ? *reinterpret_cast<const int *>(src) : 0;
-        r[i] = v;
+        for (int d = 0; d < 4; ++d) {
+          if (tap_addr(ent[i][d], s, src)) m |= 1u << (4 * i + d);
+          v[d] = *reinterpret_cast<const int *>(src);
+        }
+        r[S][i] = v;
+      } else {
+        static_assert(TAPB == 16 || TAPB == 32, "tap width");
+        const bool ok = tap_addr(ent[i][0], s, src);
+        if (ok) m |= 0xFu << (4 * i);
+        r[S][i] = *reinterpret_cast<const v4i *>(src + ((TAPB == 32 && ok) ? (g & 1) * 16 : 0));
       }
     }
+    okm[S] = m;
   }
 
+  template <int S>
   __device__ __forceinline__ void commit(char *tile) {
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      v4i v = r[i];
+      v4i v;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) v[d] = (okm[S] >> (4 * i + d)) & 1 ? r[S][i][d] : 0;
       if (XOR80) v ^= (int)0x80808080;
       const int row = prow + (i % PPT) * NT;
       *reinterpret_cast<v4i *>(tile + lds_off<BKB>(row, (i / PPT) * TPS + tq)) = v;

@@ -10,11 +10,13 @@
 // (accumulator columns, spread over lanes):  lane l, register r of a 32x32 block hold
 //   x = 8*(r/4) + 4*(l/32) + r%4,   y = l%32.
 //
-// Pipeline: global -> registers (one stage ahead) -> LDS (double buffered) -> MFMA, one
-// workgroup barrier per stage.
+// Pipeline: global -> registers (one stage ahead) -> LDS (double buffered) -> fragments (double
+// buffered in registers) -> MFMA, one workgroup barrier per stage.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <type_traits>
 
 namespace unit {
 
@@ -80,17 +82,19 @@ struct Tile {
   static_assert(BX % (WX * 32) == 0 && BY % (WY * 32) == 0, "wave tile is a multiple of 32x32");
 };
 
-// Workgroup id -> tile coordinates.  Workgroups are dealt round-robin to the 8 XCDs, each with
+// Workgroup id -> (tile, k-split).  Workgroups are dealt round-robin to the 8 XCDs, each with
 // its own L2: ids congruent mod 8 share an XCD, so they are given consecutive logical ids, and
 // logical ids walk the tile grid in panels `ph` X-tiles tall so that an XCD's working set is a
-// compact patch of the grid.
+// compact patch of the grid.  The k-splits of one tile are adjacent logical ids.
 struct GridMap {
-  int gx, gy, ph, total;
-  __device__ __forceinline__ void locate(int bid, int &bx, int &by) const {
+  int gx, gy, ph, splits, total;  // total = gx * gy * splits
+  __device__ __forceinline__ void locate(int bid, int &bx, int &by, int &split) const {
     constexpr int NXCD = 8;
     int per = total / NXCD, rem = total % NXCD;
     int xcd = bid % NXCD, idx = bid / NXCD;
     int logical = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    split = logical % splits;
+    logical /= splits;
     int panel_sz = ph * gy;
     int panel = logical / panel_sz, within = logical - panel * panel_sz;
     int rows = gx - panel * ph;
@@ -106,19 +110,28 @@ enum { WS_NONE = 0, WS_X = 1, WS_Y = 2 };
 // WS selects which operand is the s8 weight whose per-row byte sums are accumulated on the side
 // (v_dot4 against 0x01010101): the u8 operand is staged as (u8 ^ 0x80) = u8 - 128 reinterpreted
 // as s8, because the MFMA int8 path multiplies signed by signed, and the epilogue adds back
-// 128 * sum_k w[k].
+// 128 * sum_k w[k].  With k-splits each workgroup adds the correction of its own k-range.
+//
+// Schedule of one pipeline stage (KK = BKB / 32 MFMA k-steps, fragments double-buffered in
+// registers):   ds_write stage+1 | global_load stage+2 | for kk: ds_read frags(kk+1), MFMA(kk) |
+// before the last k-step: barrier, ds_read frags(0) of the next stage, then the last MFMAs --
+// so LDS latency and the barrier skew are covered by MFMA work of the same wave.
 template <class Op, class T, class XL, class YL, class Epi, int WS>
 __global__ __launch_bounds__(T::NT) void mma_kernel(typename XL::Params xp, typename YL::Params yp,
-                                                    typename Epi::Params ep, int nk, GridMap gm) {
+                                                    typename Epi::Params ep, int nk_total, GridMap gm) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   const int t = threadIdx.x;
   const int lane = t & 63, wave = t >> 6;
   const int wx = wave % T::WX, wy = wave / T::WX;
   const int l32 = lane & 31, half = lane >> 5;
+  constexpr int KK = T::BKB / 32;
+  static_assert(KK % 2 == 0, "fragment double buffering needs an even number of k-steps");
 
-  int bx, by;
-  gm.locate(blockIdx.x, bx, by);
+  int bx, by, split;
+  gm.locate(blockIdx.x, bx, by, split);
   const int x0 = bx * T::BX, y0 = by * T::BY;
+  // this workgroup's stages: [kb, ke)
+  const int kb = (int)((long)nk_total * split / gm.splits), ke = (int)((long)nk_total * (split + 1) / gm.splits);
 
   XL xl;
   YL yl;
@@ -144,57 +157,112 @@ __global__ __launch_bounds__(T::NT) void mma_kernel(typename XL::Params xp, type
   // 32-row block starts at a multiple of 32, so one mask serves all blocks of a lane
   const int xrow = wx * (T::TX * 32) + l32, yrow = wy * (T::TY * 32) + l32;
   const int xsw = swz<T::BKB>(xrow), ysw = swz<T::BKB>(yrow);
+  const int xbase = xrow * T::BKB, ybase = T::XBYTES + yrow * T::BKB;
 
-  if (XL::kNeedsSync || YL::kNeedsSync) __syncthreads();  // tap tables visible
-  xl.fetch(0);
-  yl.fetch(0);
-  xl.commit(lds);
-  yl.commit(lds + T::XBYTES);
-  if (nk > 1) {
-    xl.fetch(1);
-    yl.fetch(1);
-  }
-  __syncthreads();
-
-  for (int kt = 0; kt < nk; ++kt) {
-    char *cur = lds + (kt & 1) * T::STAGE;
-    char *nxt = lds + ((kt & 1) ^ 1) * T::STAGE;
-    if (kt + 1 < nk) {  // registers hold stage kt+1
-      xl.commit(nxt);
-      yl.commit(nxt + T::XBYTES);
-    }
-    if (kt + 2 < nk) {
-      xl.fetch(kt + 2);
-      yl.fetch(kt + 2);
-    }
-    const char *xs = cur + xrow * T::BKB, *ys = cur + T::XBYTES + yrow * T::BKB;
+  v4i xf[2][T::TX], yf[2][T::TY];
+  auto load_frags = [&](const char *stage, int kk, int slot) __attribute__((always_inline)) {
 #pragma unroll
-    for (int kk = 0; kk < T::BKB / 32; ++kk) {
-      v4i xf[T::TX], yf[T::TY];
+    for (int i = 0; i < T::TX; ++i)
+      xf[slot][i] = *reinterpret_cast<const v4i *>(stage + xbase + i * 32 * T::BKB + (((2 * kk + half) ^ xsw) << 4));
+#pragma unroll
+    for (int j = 0; j < T::TY; ++j)
+      yf[slot][j] = *reinterpret_cast<const v4i *>(stage + ybase + j * 32 * T::BKB + (((2 * kk + half) ^ ysw) << 4));
+  };
+  auto mma_step = [&](int slot) __attribute__((always_inline)) {
+    if constexpr (WS == WS_X) {
 #pragma unroll
       for (int i = 0; i < T::TX; ++i)
-        xf[i] = *reinterpret_cast<const v4i *>(xs + i * 32 * T::BKB + (((2 * kk + half) ^ xsw) << 4));
+#pragma unroll
+        for (int d = 0; d < 4; ++d) wsx[i] = __builtin_amdgcn_sdot4(xf[slot][i][d], 0x01010101, wsx[i], false);
+    }
+    if constexpr (WS == WS_Y) {
 #pragma unroll
       for (int j = 0; j < T::TY; ++j)
-        yf[j] = *reinterpret_cast<const v4i *>(ys + j * 32 * T::BKB + (((2 * kk + half) ^ ysw) << 4));
-      if constexpr (WS == WS_X) {
 #pragma unroll
-        for (int i = 0; i < T::TX; ++i)
+        for (int d = 0; d < 4; ++d) wsy[j] = __builtin_amdgcn_sdot4(yf[slot][j][d], 0x01010101, wsy[j], false);
+    }
 #pragma unroll
-          for (int d = 0; d < 4; ++d) wsx[i] = __builtin_amdgcn_sdot4(xf[i][d], 0x01010101, wsx[i], false);
+    for (int i = 0; i < T::TX; ++i)
+#pragma unroll
+      for (int j = 0; j < T::TY; ++j) acc[i][j] = Op::mma(xf[slot][i], yf[slot][j], acc[i][j]);
+  };
+
+  // One pipeline stage.  U is the register slot that holds stage kt+1 (stages rotate through PF
+  // slots, so PF stages of global loads are in flight).  NEXT: stage kt+1 exists (write it to
+  // LDS, and after the barrier pre-load its first fragments); NEXTPF: stage kt+1+PF exists (fetch
+  // it into the slot just freed).
+  constexpr int PF = XL::kPF;
+  static_assert(XL::kPF == YL::kPF, "both operands use the same prefetch depth");
+  auto stage = [&](int kt, int par, auto slot, bool next, bool nextpf) __attribute__((always_inline)) {
+    constexpr int U = decltype(slot)::value;
+    char *cur = lds + par * T::STAGE;
+    char *nxt = lds + (par ^ 1) * T::STAGE;
+    if (next) {
+      xl.template commit<U>(nxt);
+      yl.template commit<U>(nxt + T::XBYTES);
+    }
+    if (nextpf) {
+      xl.template fetch<U>(kt + 1 + PF);
+      yl.template fetch<U>(kt + 1 + PF);
+    }
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      if (kk + 1 < KK) {
+        load_frags(cur, kk + 1, (kk + 1) & 1);
+        mma_step(kk & 1);
+      } else {
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();  // everyone has read `cur` and written `nxt`
+        if (next) load_frags(nxt, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        mma_step(kk & 1);
       }
-      if constexpr (WS == WS_Y) {
-#pragma unroll
-        for (int j = 0; j < T::TY; ++j)
-#pragma unroll
-          for (int d = 0; d < 4; ++d) wsy[j] = __builtin_amdgcn_sdot4(yf[j][d], 0x01010101, wsy[j], false);
+    }
+  };
+  // stage kt with the slot rotation resolved at compile time for PF consecutive stages
+  auto stages_pf = [&](int kt, int par, auto steady) __attribute__((always_inline)) {
+    auto one = [&](auto u) __attribute__((always_inline)) {
+      constexpr int UU = decltype(u)::value;
+      const int k = kt + UU;
+      if constexpr (decltype(steady)::value) {
+        stage(k, (par + UU) & 1, std::integral_constant<int, (UU + 1) % PF>{}, true, true);
+      } else {
+        if (k < ke) stage(k, (par + UU) & 1, std::integral_constant<int, (UU + 1) % PF>{}, k + 1 < ke, k + 1 + PF < ke);
       }
-#pragma unroll
-      for (int i = 0; i < T::TX; ++i)
-#pragma unroll
-        for (int j = 0; j < T::TY; ++j) acc[i][j] = Op::mma(xf[i], yf[j], acc[i][j]);
+    };
+    one(std::integral_constant<int, 0>{});
+    if constexpr (PF > 1) one(std::integral_constant<int, 1>{});
+    if constexpr (PF > 2) one(std::integral_constant<int, 2>{});
+    if constexpr (PF > 3) one(std::integral_constant<int, 3>{});
+  };
+  static_assert(PF >= 1 && PF <= 4, "prefetch depth 1..4");
+
+  if (XL::kNeedsSync || YL::kNeedsSync) __syncthreads();  // tap tables visible
+  if (kb < ke) {
+    // prologue: PF stages in flight, the first one staged into LDS
+    xl.template fetch<0>(kb);
+    yl.template fetch<0>(kb);
+    if constexpr (PF > 1) {
+      if (kb + 1 < ke) { xl.template fetch<1 % PF>(kb + 1); yl.template fetch<1 % PF>(kb + 1); }
+    }
+    if constexpr (PF > 2) {
+      if (kb + 2 < ke) { xl.template fetch<2 % PF>(kb + 2); yl.template fetch<2 % PF>(kb + 2); }
+    }
+    if constexpr (PF > 3) {
+      if (kb + 3 < ke) { xl.template fetch<3 % PF>(kb + 3); yl.template fetch<3 % PF>(kb + 3); }
+    }
+    xl.template commit<0>(lds);
+    yl.template commit<0>(lds + T::XBYTES);
+    if (kb + PF < ke) {
+      xl.template fetch<0>(kb + PF);
+      yl.template fetch<0>(kb + PF);
     }
     __syncthreads();
+    load_frags(lds, 0, 0);
+    int kt = kb, par = 0;
+    // steady state: every stage of the group has a successor and a stage PF+1 ahead to fetch
+    for (; kt + 2 * PF < ke; kt += PF, par = (par + PF) & 1) stages_pf(kt, par, std::true_type{});
+    for (; kt < ke; kt += PF, par = (par + PF) & 1) stages_pf(kt, par, std::false_type{});
   }
 
   // the two 32-lane halves hold the sums of the two 16-byte k-chunks of every MFMA step
@@ -207,8 +275,15 @@ __global__ __launch_bounds__(T::NT) void mma_kernel(typename XL::Params xp, type
     for (int j = 0; j < T::TY; ++j) wsy[j] += __shfl_xor(wsy[j], 32);
   }
 
+  // the last barrier of the K loop came after every LDS read: the tiles are free for the epilogue
   Epi::template store<T>(ep, acc, wsx, wsy, x0 + wx * (T::TX * 32), y0 + wy * (T::TY * 32), lane, wave,
-                         lds);
+                         lds, gm.splits > 1);
+}
+
+// zero fill for outputs accumulated with atomics (k-splits): 16 bytes per thread
+static __global__ __launch_bounds__(256) void zero_fill(v4i *dst, size_t n16) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n16) dst[i] = v4i{0, 0, 0, 0};
 }
 
 }  // namespace unit

@@ -1,0 +1,204 @@
+// GEMM kernel whose operand tiles go global -> LDS directly (global_load_lds_dwordx4, no VGPR
+// round trip) through a ring of NSTAGE LDS buffers, so NSTAGE-1 stages of loads are in flight
+// while one is consumed.  Both operands must be K-contiguous rows (A (M, K) and W (N, K)) and the
+// reduction a whole number of stages; everything else uses mma_kernel.
+//
+// A wave-level direct load writes 64 lanes x 16 bytes = 1 KiB of consecutive LDS, so lane i
+// fetches the global chunk that belongs at LDS position i of that KiB: LDS rows keep the same
+// XOR-swizzled [row][BKB] layout the MFMA fragment reads of mma_kernel use.  The u8 operand
+// cannot be shifted to s8 on the way, so it is shifted after the fragment read (4 v_xor per
+// fragment).
+#pragma once
+#include "mma_core.hpp"
+
+namespace unit {
+
+typedef const __attribute__((address_space(1))) void *gptr_t;
+typedef __attribute__((address_space(3))) void *lptr_t;
+
+// s_waitcnt vmcnt(n) only (expcnt / lgkmcnt fields left at "no wait"), gfx9 encoding
+#define UNIT_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
+
+struct DmaParams {
+  const char *x;  // X rows (first MFMA operand), K-contiguous
+  const char *y;  // Y rows
+  int xrows, yrows;
+  int ld;         // bytes per row (both operands)
+};
+
+template <class Op, class T, int NSTAGE, class Epi, int WS, bool XOR_X>
+__global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Epi::Params ep, int nk, GridMap gm) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  const int t = threadIdx.x;
+  const int lane = t & 63, wave = t >> 6;
+  const int wx = wave % T::WX, wy = wave / T::WX;
+  const int l32 = lane & 31, half = lane >> 5;
+  constexpr int KK = T::BKB / 32, CPR = T::CPR, NW = T::NT / 64;
+  constexpr int RPL = 64 / CPR;                  // rows per wave-level load (1 KiB)
+  constexpr int XL = T::BX / RPL / NW;           // loads per wave per stage, X tile
+  constexpr int YL = T::BY / RPL / NW;
+  static_assert(T::BX % (RPL * NW) == 0 && T::BY % (RPL * NW) == 0, "tile rows split evenly over the waves");
+  static_assert(KK % 2 == 0, "fragment double buffering needs an even number of k-steps");
+  constexpr int LPS = XL + YL;                   // loads per wave per stage
+
+  int bx, by, split;
+  gm.locate(blockIdx.x, bx, by, split);
+  const int x0 = bx * T::BX, y0 = by * T::BY;
+
+  // per-lane source offsets: lane -> (row, slot) of its KiB, chunk = slot ^ swizzle(row)
+  u32 xoff[XL], yoff[YL];
+  const int lrow = lane / CPR, slot = lane % CPR;
+#pragma unroll
+  for (int i = 0; i < XL; ++i) {
+    const int row = (wave * XL + i) * RPL + lrow;
+    int g = x0 + row;
+    g = g < p.xrows ? g : p.xrows - 1;
+    xoff[i] = (u32)g * (u32)p.ld + ((slot ^ swz<T::BKB>(row)) << 4);
+  }
+#pragma unroll
+  for (int i = 0; i < YL; ++i) {
+    const int row = (wave * YL + i) * RPL + lrow;
+    int g = y0 + row;
+    g = g < p.yrows ? g : p.yrows - 1;
+    yoff[i] = (u32)g * (u32)p.ld + ((slot ^ swz<T::BKB>(row)) << 4);
+  }
+
+  auto issue = [&](int kt) {
+    char *buf = lds + (kt % NSTAGE) * T::STAGE;
+    const char *xs = p.x + (size_t)kt * T::BKB, *ys = p.y + (size_t)kt * T::BKB;
+#pragma unroll
+    for (int i = 0; i < XL; ++i)
+      __builtin_amdgcn_global_load_lds((gptr_t)(xs + xoff[i]), (lptr_t)(buf + (wave * XL + i) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int i = 0; i < YL; ++i)
+      __builtin_amdgcn_global_load_lds((gptr_t)(ys + yoff[i]), (lptr_t)(buf + T::XBYTES + (wave * YL + i) * 1024), 16,
+                                       0, 0);
+  };
+
+  typename Op::acc_t acc[T::TX][T::TY];
+#pragma unroll
+  for (int i = 0; i < T::TX; ++i)
+#pragma unroll
+    for (int j = 0; j < T::TY; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+  int wsx[T::TX], wsy[T::TY];
+#pragma unroll
+  for (int i = 0; i < T::TX; ++i) wsx[i] = 0;
+#pragma unroll
+  for (int j = 0; j < T::TY; ++j) wsy[j] = 0;
+
+  const int xrow = wx * (T::TX * 32) + l32, yrow = wy * (T::TY * 32) + l32;
+  const int xsw = swz<T::BKB>(xrow), ysw = swz<T::BKB>(yrow);
+  const int xbase = xrow * T::BKB, ybase = T::XBYTES + yrow * T::BKB;
+
+  v4i xf[2][T::TX], yf[2][T::TY];
+  // fragment i of the step's read list: X0, Y0..Y(TY-1), X1..X(TX-1) -- the first MFMA needs
+  // only the first two
+  auto load_one = [&](const char *stage, int kk, int s, int idx) {
+    const int cx = ((2 * kk + half) ^ xsw) << 4, cy = ((2 * kk + half) ^ ysw) << 4;
+    if (idx == 0)
+      xf[s][0] = *reinterpret_cast<const v4i *>(stage + xbase + cx);
+    else if (idx <= T::TY)
+      yf[s][idx - 1] = *reinterpret_cast<const v4i *>(stage + ybase + (idx - 1) * 32 * T::BKB + cy);
+    else
+      xf[s][idx - T::TY] = *reinterpret_cast<const v4i *>(stage + xbase + (idx - T::TY) * 32 * T::BKB + cx);
+  };
+  auto load_frags = [&](const char *stage, int kk, int s) {
+#pragma unroll
+    for (int i = 0; i < T::TX + T::TY; ++i) load_one(stage, kk, s, i);
+  };
+  auto issue_one = [&](int kt, int i) {
+    char *buf = lds + (kt % NSTAGE) * T::STAGE;
+    const char *xs = p.x + (size_t)kt * T::BKB, *ys = p.y + (size_t)kt * T::BKB;
+    if (i < XL)
+      __builtin_amdgcn_global_load_lds((gptr_t)(xs + xoff[i]), (lptr_t)(buf + (wave * XL + i) * 1024), 16, 0, 0);
+    else
+      __builtin_amdgcn_global_load_lds((gptr_t)(ys + yoff[i - XL]),
+                                       (lptr_t)(buf + T::XBYTES + (wave * YL + (i - XL)) * 1024), 16, 0, 0);
+  };
+
+  // One k-step with a fixed instruction order: every MFMA is followed by one slice of the
+  // step's other work (a fragment read for the next step, a direct load for a later stage, the
+  // u8 -> s8 shift of the next X fragment, one weight-sum dot) and a scheduling fence, because
+  // with one wave per SIMD only instructions placed between two MFMAs overlap with them.
+  //   s: fragment slot consumed;  rd_stage/rd_kk: where the next step's fragments come from
+  //   (nullptr: none);  issue_kt >= 0: stage to fetch with direct loads.
+  auto step = [&](int s, const char *rd_stage, int rd_kk, int issue_kt, auto has_read, auto has_issue) {
+    constexpr int NM = T::TX * T::TY, NF = T::TX + T::TY;
+    if constexpr (XOR_X) xf[s][0] ^= (int)0x80808080;
+#pragma unroll
+    for (int m = 0; m < NM; ++m) {
+      const int i = m / T::TY, j = m % T::TY;
+      acc[i][j] = Op::mma(xf[s][i], yf[s][j], acc[i][j]);
+      if constexpr (decltype(has_read)::value) {
+        if (m < NF) load_one(rd_stage, rd_kk, s ^ 1, m);
+      }
+      if constexpr (decltype(has_issue)::value) {
+        if (m >= NM - LPS) issue_one(issue_kt, m - (NM - LPS));
+      }
+      if constexpr (XOR_X) {
+        if (j == T::TY - 1 && i + 1 < T::TX) xf[s][i + 1] ^= (int)0x80808080;
+      }
+      if constexpr (WS == WS_Y) {
+        // TY fragments x 4 dwords spread over the first 4*TY MFMAs
+        if (m < 4 * T::TY) wsy[m / 4] = __builtin_amdgcn_sdot4(yf[s][m / 4][m % 4], 0x01010101, wsy[m / 4], false);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  static_assert(T::TX * T::TY >= LPS && T::TX * T::TY >= T::TX + T::TY && T::TX * T::TY >= 4 * T::TY,
+                "not enough MFMAs per k-step to carry the step's other work");
+
+  // One stage.  ISSUE: stage kt + NSTAGE exists and is fetched into the buffer this stage
+  // frees; STEADY: NSTAGE-1 younger stages are in flight when the barrier is reached (else
+  // wait for everything); NEXT: stage kt + 1 exists.
+  auto stage = [&](int kt, auto issue_next, auto steady, auto next) {
+    const char *cur = lds + (kt % NSTAGE) * T::STAGE;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      if (kk + 1 < KK) {
+        step(kk & 1, cur, kk + 1, -1, std::true_type{}, std::false_type{});
+      } else {
+        // stage kt+1 must have landed; stages kt+2 .. kt+NSTAGE-1 may stay in flight
+        if constexpr (decltype(steady)::value)
+          UNIT_WAIT_VMCNT((NSTAGE - 2) * LPS);
+        else
+          UNIT_WAIT_VMCNT(0);
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's reads of `cur` are done
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        // every wave has read stage kt: its buffer takes stage kt + NSTAGE
+        step(kk & 1, lds + ((kt + 1) % NSTAGE) * T::STAGE, 0, kt + NSTAGE, next, issue_next);
+      }
+    }
+  };
+  using yes = std::integral_constant<bool, true>;
+  using no = std::integral_constant<bool, false>;
+
+  // prologue: fill the ring
+#pragma unroll
+  for (int s = 0; s < NSTAGE; ++s)
+    if (s < nk) issue(s);
+  // stage 0 landed?  (the NSTAGE-1 younger stages may still be in flight)
+  if (nk >= NSTAGE)
+    UNIT_WAIT_VMCNT((NSTAGE - 1) * LPS);
+  else
+    UNIT_WAIT_VMCNT(0);
+  __builtin_amdgcn_s_barrier();
+  load_frags(lds, 0, 0);
+
+  int kt = 0;
+  for (; kt + NSTAGE < nk; ++kt) stage(kt, yes{}, yes{}, yes{});
+  for (; kt + 1 < nk; ++kt) stage(kt, no{}, no{}, yes{});
+  if (kt < nk) stage(kt, no{}, no{}, no{});
+
+  if constexpr (WS == WS_Y) {
+#pragma unroll
+    for (int j = 0; j < T::TY; ++j) wsy[j] += __shfl_xor(wsy[j], 32);
+  }
+  Epi::template store<T>(ep, acc, wsx, wsy, x0 + wx * (T::TX * 32), y0 + wy * (T::TY * 32), lane, wave, lds,
+                         gm.splits > 1);
+}
+
+}  // namespace unit

@@ -1,0 +1,147 @@
+"""Kernel-variant tuner for the int8 convolution: the counterpart of the reference's tuning loop
+(apps/cpu/kernel/conv2d.py:37-83 tries schedule candidates one by one, keeps the fastest and
+appends it to cpu-tune.log; python/tensorizer/tune.py:20-31 reads that log back into a table
+keyed by (ashape, bshape, strides)).
+
+Here the candidates are the tile variants compiled into libunit_amd.so.  For every layer shape
+each variant is run through the C ABI, checked bit for bit against the library's default choice,
+and timed with HIP events; the fastest goes into unit_amd/csrc/tuned_conv_i8.inc, which the
+library's planner consults first (rebuild after tuning).  Needs an MI355X.
+
+    python -m unit_amd.tune [--nets resnet50:32,resnet18:1] [--iters 20] [--write]
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+
+NUM_VARIANTS = 26  # kConvTiles in csrc/conv_plan.hpp
+
+
+def _shapes(spec):
+    from . import workloads as WL
+    nets = {"resnet50": WL.RESNET50, "resnet18": WL.RESNET18, "single": (WL.SINGLE_CONV,)}
+    out = []
+    for item in spec.split(","):
+        name, batch = item.split(":")
+        for s in nets[name]:
+            out.append((name, int(batch), s))
+    return out
+
+
+def tune(spec, iters=20, verbose=True):
+    import torch
+
+    from . import _lib, last_variant
+    from . import workloads as WL
+
+    dev = torch.device("cuda:0")
+    L = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def time_us(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / iters
+
+    saved = {k: os.environ.get(k) for k in ("UNIT_AMD_CONV_VARIANT", "UNIT_AMD_CONV_SPLITK")}
+    results = []
+    seen = set()
+    try:
+        for net, batch, s in _shapes(spec):
+            cb = WL.channel_block(s.C)
+            cp = -(-s.C // cb) * cb
+            oh, ow = WL.out_hw(s)
+            key = (batch * oh * ow, s.K, cp, s.KH, s.KW, s.stride)
+            if key in seen:
+                continue
+            seen.add(key)
+            data = torch.randint(0, 256, (batch, cp // cb, s.H, s.W, cb), dtype=torch.uint8, device=dev)
+            wt = torch.randint(-128, 128, (s.K // 16, cp // cb, s.KH, s.KW, cb // 4, 16, 4), dtype=torch.int8, device=dev)
+            out = torch.empty((batch, s.K // 16, oh, ow, 16), dtype=torch.int32, device=dev)
+            desc = _lib.ConvDesc(batch, cp, s.H, s.W, s.K, s.KH, s.KW, s.stride, s.stride, s.pad, s.pad, s.pad, s.pad,
+                                 1, 1, cb)
+
+            def call():
+                return L.unit_conv2d_nchwc_u8s8s32(ctypes.byref(desc), data.data_ptr(), wt.data_ptr(), out.data_ptr(),
+                                                   stream)
+
+            os.environ["UNIT_AMD_CONV_VARIANT"] = "0"
+            os.environ["UNIT_AMD_CONV_SPLITK"] = "0"
+            _lib.check(call())
+            torch.cuda.synchronize()
+            ref = out.clone()
+            best = (time_us(call), -1, last_variant())
+            default_us = best[0]
+            for v in range(NUM_VARIANTS):
+                for splits in (1, 2, 4, 8, 16, 32):
+                    os.environ["UNIT_AMD_CONV_VARIANT"] = str(v + 1)
+                    os.environ["UNIT_AMD_CONV_SPLITK"] = str(splits)
+                    out.fill_(-7)
+                    if call() != 0:  # variant cannot run this shape (LDS budget)
+                        break
+                    torch.cuda.synchronize()
+                    name = last_variant()
+                    if int(name.rsplit("_s", 1)[1]) != splits:
+                        break  # clamped to the number of stages: already measured
+                    if not torch.equal(out, ref):
+                        raise RuntimeError(f"variant {v} ({name}) disagrees with the default on {s.name}")
+                    us = time_us(call)
+                    if us < best[0]:
+                        best = (us, v, name, splits)
+                    if splits * key[0] * s.K > 256 * 256 * 256:
+                        break  # the grid already covers the chip: more k-splits only add atomics
+            results.append(dict(net=net, batch=batch, layer=s.name, key=key, variant=best[1], us=best[0],
+                                default_us=default_us, kernel=best[2], splits=best[3] if len(best) > 3 else 1))
+            if verbose:
+                print(f"{net:9s} b{batch:<3d} {s.name:22s} default {default_us:7.1f} us  best {best[0]:7.1f} us  {best[2]}",
+                      flush=True)
+    finally:
+        for k, v in saved.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
+    return results
+
+
+def write_table(results, path):
+    lines = []
+    for r in results:
+        if r["variant"] < 0:
+            continue  # the heuristic's own choice was the fastest
+        npix, k, c, kh, kw, sh = r["key"]
+        lines.append(f"    {{{npix}, {k}, {c}, {kh}, {kw}, {sh}, {r['variant']}, {r['splits']}}},  // {r['net']} b{r['batch']} "
+                     f"{r['layer']}: {r['us']:.1f} us ({r['kernel']})\n")
+    with open(path, "w") as f:
+        f.writelines(lines)
+    return len(lines)
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--nets", default="resnet50:32,resnet18:1,single:1")
+    ap.add_argument("--iters", type=int, default=20)
+    ap.add_argument("--write", action="store_true", help="rewrite csrc/tuned_conv_i8.inc")
+    ap.add_argument("--table", default=None, help="write the table here instead of csrc/tuned_conv_i8.inc")
+    ap.add_argument("--json", default=None, help="also dump the raw results here")
+    args = ap.parse_args()
+    results = tune(args.nets, args.iters)
+    if args.json:
+        json.dump(results, open(args.json, "w"), indent=1)
+    if args.write or args.table:
+        path = args.table or os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "tuned_conv_i8.inc")
+        n = write_table(results, path)
+        print(f"wrote {n} entries to {path}; rebuild with `make -C {os.path.dirname(path)}`")
+
+
+if __name__ == "__main__":
+    sys.exit(main())
