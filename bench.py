@@ -198,6 +198,87 @@ def main():
                     pct_f16_peak=round(100 * gemm_ops / us_f / 1e6 / PEAK_F16_TFLOPS, 2), kernel=v_f,
                     max_rel_err=f16_err, tolerance=1e-2)
 
+    # ------------------------------------------------------------------ secondary legs (BASELINE configs 0, 3, 4-fp16, layouts)
+    def conv_i8_leg(shapes, batch, iters):
+        rows, tot_us, tot_ops = [], 0.0, 0.0
+        for i, s in enumerate(shapes):
+            cb = WL.channel_block(s.C)
+            cp = -(-s.C // cb) * cb
+            d = dev_t(rng.uniform_u8((batch, cp // cb, s.H, s.W, cb), 3000 + i))
+            w = dev_t(rng.uniform_s8((s.K // 16, cp // cb, s.KH, s.KW, cb // 4, 16, 4), 4000 + i))
+            oh, ow = WL.out_hw(s)
+            o = torch.empty((batch, s.K // 16, oh, ow, 16), dtype=torch.int32, device=dev)
+            desc = _lib.ConvDesc(batch, cp, s.H, s.W, s.K, s.KH, s.KW, s.stride, s.stride, s.pad, s.pad, s.pad, s.pad,
+                                 1, 1, cb)
+            f = lambda: _lib.check(L.unit_conv2d_nchwc_u8s8s32(ctypes.byref(desc), d.data_ptr(), w.data_ptr(),
+                                                               o.data_ptr(), stream))
+            us = time_us(f, iters)
+            ops = 2 * WL.macs(s, batch)
+            rows.append(dict(layer=s.name, us=round(us, 2), tops=round(ops / us / 1e6, 2), kernel=U.last_variant()))
+            tot_us += us * s.count
+            tot_ops += ops * s.count
+        return rows, tot_us, tot_ops
+
+    r18_rows, r18_us, r18_ops = conv_i8_leg(WL.RESNET18, 1, 30)
+    resnet18_b1 = dict(workload="ResNet-18 v1 conv layers, batch 1, int8 (BASELINE configs[3])",
+                       stack_us=round(r18_us, 1), tops=round(r18_ops / r18_us / 1e6, 2), layers=r18_rows)
+    single_rows, _, _ = conv_i8_leg((WL.SINGLE_CONV,), 1, 50)
+    single_conv = dict(workload="N=1 C=64 56x56 K=64 3x3 s1 p1 NCHW16c (BASELINE configs[0])", **single_rows[0],
+                       reference_us=24.27, reference_source="cpu-tune.log:160 (x86 VNNI, hardware unstated)")
+
+    # fp16 variant of the ResNet-50 b32 sweep: valid convolution on pre-padded NCHW16c inputs
+    f16_rows, f16_us, f16_flops = [], 0.0, 0.0
+    for i, s in enumerate(WL.RESNET50):
+        if s.C % 16:
+            continue  # the fp16 operator needs C % 16 == 0 (the 3-channel stem has no NCHW16c form)
+        hp, wp_ = s.H + 2 * s.pad, s.W + 2 * s.pad
+        a = torch.randn((BATCH, s.C // 16, hp, wp_, 16), dtype=torch.float16, device=dev)
+        b = torch.randn((s.K // 16, s.C // 16, s.KH, s.KW, 16, 16), dtype=torch.float16, device=dev) * 0.05
+        oh, ow = WL.out_hw(s)
+        o = torch.empty((BATCH, s.K // 16, oh, ow, 16), dtype=torch.float32, device=dev)
+        desc = _lib.ConvDesc(BATCH, s.C, hp, wp_, s.K, s.KH, s.KW, s.stride, s.stride, 0, 0, 0, 0, 1, 1, 16)
+        f = lambda: _lib.check(L.unit_conv2d_nchw16c_f16f32(ctypes.byref(desc), a.data_ptr(), b.data_ptr(),
+                                                            o.data_ptr(), stream))
+        us = time_us(f, 20)
+        flops = 2 * WL.macs(s, BATCH)
+        f16_rows.append(dict(layer=s.name, us=round(us, 2), tflops=round(flops / us / 1e6, 1),
+                             pct_f16_peak=round(100 * flops / us / 1e6 / PEAK_F16_TFLOPS, 2), kernel=U.last_variant()))
+        f16_us += us * s.count
+        f16_flops += flops * s.count
+    conv_fp16 = dict(workload="ResNet-50 v1 conv layers except the stem, batch 32, fp16 -> fp32 (BASELINE configs[4], "
+                              "fp16 variant)", stack_us=round(f16_us, 1), tflops=round(f16_flops / f16_us / 1e6, 1),
+                     layers=f16_rows)
+
+    # layout transforms / pre-packs: bytes read + written over time
+    x8 = torch.randint(0, 256, (BATCH, 256, 56, 56), dtype=torch.uint8, device=dev)
+    o32 = torch.empty((BATCH, 16, 56, 56, 16), dtype=torch.int32, device=dev)
+    w33 = torch.randint(-128, 128, (512, 512, 3, 3), dtype=torch.int8, device=dev)
+    layout = {}
+    us = time_us(lambda: U.pack_nchwc(x8, 16), 20)
+    layout["pack_nchw16c_u8_32x256x56x56"] = dict(us=round(us, 2), gbs=round(2 * x8.numel() / us / 1e3, 1))
+    us = time_us(lambda: U.unpack_nchwc(o32), 20)
+    layout["unpack_nchw16c_i32_32x256x56x56"] = dict(us=round(us, 2), gbs=round(2 * o32.numel() * 4 / us / 1e3, 1))
+    us = time_us(lambda: U.prepack_conv_weight(w33, 16), 20)
+    layout["prepack_conv_weight_512x512x3x3"] = dict(us=round(us, 2), gbs=round(2 * w33.numel() / us / 1e3, 1))
+    us = time_us(lambda: U.prepack_dense_weight(w8), 20)
+    layout["prepack_dense_weight_4096x4096"] = dict(us=round(us, 2), gbs=round(2 * w8.numel() / us / 1e3, 1))
+
+    # register-only MFMA throughput of this box (no memory traffic): what the silicon sustains
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    probe = {}
+    for f16, key, per in ((0, "int8_tops", 65536.0), (1, "fp16_tflops", 32768.0)):
+        blocks, iters = 512, 4000
+        L.unit_mfma_peak(f16, blocks, 200, sink.data_ptr(), stream)
+        us = time_us(lambda: _lib.check(L.unit_mfma_peak(f16, blocks, iters, sink.data_ptr(), stream)), 3, warm=1)
+        probe[key] = round(blocks * 16 * iters * per / us / 1e6, 1)
+
+    # HBM traffic of the dominant kernel, when a counter run has been recorded for it
+    try:
+        traffic = json.load(open(os.path.join(ROOT, "profiles", "traffic.json")))
+        roofline["traffic"] = traffic.get(roofline["layer"])
+    except (OSError, ValueError):
+        pass
+
     # ------------------------------------------------------------------ CPU baseline + bit-exactness
     cpu_baseline = None
     bit_exact = None
@@ -258,6 +339,11 @@ def main():
         "cpu_baseline": cpu_baseline,
         "gemm_int8_4096": gemm_i8,
         "gemm_fp16_4096": gemm_f16,
+        "mfma_probe": probe,
+        "single_conv": single_conv,
+        "resnet18_b1": resnet18_b1,
+        "conv_fp16_resnet50_b32": conv_fp16,
+        "layout_kernels": layout,
         "layers": table,
     }
     print(json.dumps(line))

@@ -5,10 +5,10 @@ keyed by (ashape, bshape, strides)).
 
 Here the candidates are the tile variants compiled into libunit_amd.so.  For every layer shape
 each variant is run through the C ABI, checked bit for bit against the library's default choice,
-and timed with HIP events; the fastest goes into unit_amd/csrc/tuned_conv_i8.inc, which the
+and timed with HIP events; the fastest goes into unit_amd/csrc/tuned_conv_{i8,f16}.inc, which the
 library's planner consults first (rebuild after tuning).  Needs an MI355X.
 
-    python -m unit_amd.tune [--nets resnet50:32,resnet18:1] [--iters 20] [--write]
+    python -m unit_amd.tune [--dtype i8|f16] [--nets resnet50:32,resnet18:1] [--iters 20] [--write]
 """
 import argparse
 import ctypes
@@ -30,7 +30,7 @@ def _shapes(spec):
     return out
 
 
-def tune(spec, iters=20, verbose=True):
+def tune(spec, iters=20, verbose=True, dtype="i8"):
     import torch
 
     from . import _lib, last_variant
@@ -57,22 +57,33 @@ def tune(spec, iters=20, verbose=True):
     seen = set()
     try:
         for net, batch, s in _shapes(spec):
-            cb = WL.channel_block(s.C)
+            cb = WL.channel_block(s.C) if dtype == "i8" else 16
+            if s.C % cb and dtype != "i8":
+                continue  # the fp16 operator needs C % 16 == 0
             cp = -(-s.C // cb) * cb
             oh, ow = WL.out_hw(s)
             key = (batch * oh * ow, s.K, cp, s.KH, s.KW, s.stride)
             if key in seen:
                 continue
             seen.add(key)
-            data = torch.randint(0, 256, (batch, cp // cb, s.H, s.W, cb), dtype=torch.uint8, device=dev)
-            wt = torch.randint(-128, 128, (s.K // 16, cp // cb, s.KH, s.KW, cb // 4, 16, 4), dtype=torch.int8, device=dev)
-            out = torch.empty((batch, s.K // 16, oh, ow, 16), dtype=torch.int32, device=dev)
-            desc = _lib.ConvDesc(batch, cp, s.H, s.W, s.K, s.KH, s.KW, s.stride, s.stride, s.pad, s.pad, s.pad, s.pad,
-                                 1, 1, cb)
+            if dtype == "i8":
+                data = torch.randint(0, 256, (batch, cp // cb, s.H, s.W, cb), dtype=torch.uint8, device=dev)
+                wt = torch.randint(-128, 128, (s.K // 16, cp // cb, s.KH, s.KW, cb // 4, 16, 4), dtype=torch.int8,
+                                   device=dev)
+                out = torch.empty((batch, s.K // 16, oh, ow, 16), dtype=torch.int32, device=dev)
+                desc = _lib.ConvDesc(batch, cp, s.H, s.W, s.K, s.KH, s.KW, s.stride, s.stride, s.pad, s.pad, s.pad,
+                                     s.pad, 1, 1, cb)
+                entry = L.unit_conv2d_nchwc_u8s8s32
+            else:  # valid convolution on the pre-padded input, integer-valued data: every variant is exact
+                hp, wp = s.H + 2 * s.pad, s.W + 2 * s.pad
+                data = torch.randint(-3, 4, (batch, cp // 16, hp, wp, 16), device=dev).to(torch.float16)
+                wt = torch.randint(-3, 4, (s.K // 16, cp // 16, s.KH, s.KW, 16, 16), device=dev).to(torch.float16)
+                out = torch.empty((batch, s.K // 16, oh, ow, 16), dtype=torch.float32, device=dev)
+                desc = _lib.ConvDesc(batch, cp, hp, wp, s.K, s.KH, s.KW, s.stride, s.stride, 0, 0, 0, 0, 1, 1, 16)
+                entry = L.unit_conv2d_nchw16c_f16f32
 
             def call():
-                return L.unit_conv2d_nchwc_u8s8s32(ctypes.byref(desc), data.data_ptr(), wt.data_ptr(), out.data_ptr(),
-                                                   stream)
+                return entry(ctypes.byref(desc), data.data_ptr(), wt.data_ptr(), out.data_ptr(), stream)
 
             os.environ["UNIT_AMD_CONV_VARIANT"] = "0"
             os.environ["UNIT_AMD_CONV_SPLITK"] = "0"
@@ -82,7 +93,7 @@ def tune(spec, iters=20, verbose=True):
             best = (time_us(call), -1, last_variant())
             default_us = best[0]
             for v in range(NUM_VARIANTS):
-                for splits in (1, 2, 4, 8, 16, 32):
+                for splits in ((1, 2, 4, 8, 16, 32) if dtype == "i8" else (1,)):
                     os.environ["UNIT_AMD_CONV_VARIANT"] = str(v + 1)
                     os.environ["UNIT_AMD_CONV_SPLITK"] = str(splits)
                     out.fill_(-7)
@@ -90,7 +101,7 @@ def tune(spec, iters=20, verbose=True):
                         break
                     torch.cuda.synchronize()
                     name = last_variant()
-                    if int(name.rsplit("_s", 1)[1]) != splits:
+                    if dtype == "i8" and int(name.rsplit("_s", 1)[1]) != splits:
                         break  # clamped to the number of stages: already measured
                     if not torch.equal(out, ref):
                         raise RuntimeError(f"variant {v} ({name}) disagrees with the default on {s.name}")
@@ -130,15 +141,17 @@ def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--nets", default="resnet50:32,resnet18:1,single:1")
     ap.add_argument("--iters", type=int, default=20)
+    ap.add_argument("--dtype", default="i8", choices=["i8", "f16"])
     ap.add_argument("--write", action="store_true", help="rewrite csrc/tuned_conv_i8.inc")
     ap.add_argument("--table", default=None, help="write the table here instead of csrc/tuned_conv_i8.inc")
     ap.add_argument("--json", default=None, help="also dump the raw results here")
     args = ap.parse_args()
-    results = tune(args.nets, args.iters)
+    results = tune(args.nets, args.iters, dtype=args.dtype)
     if args.json:
         json.dump(results, open(args.json, "w"), indent=1)
     if args.write or args.table:
-        path = args.table or os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "tuned_conv_i8.inc")
+        path = args.table or os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc",
+                                          f"tuned_conv_{args.dtype}.inc")
         n = write_table(results, path)
         print(f"wrote {n} entries to {path}; rebuild with `make -C {os.path.dirname(path)}`")
 
