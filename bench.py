@@ -25,6 +25,14 @@ PEAK_INT8_TOPS = 5033.0   # MI355X dense int8 MFMA, published
 PEAK_F16_TFLOPS = 2516.0  # MI355X dense fp16 MFMA, published
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, published
 BATCH = 32
+# HBM bytes per launch (read + written) from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of
+# `bench.py --profile <layer>`, scaled by the plain-copy calibration; the summaries are
+# profiles/conv_i8_resnet50_b32_<layer>.txt and profiles/hbm_copy_calibration_128MiB.txt
+MEASURED_HBM_BYTES = {
+    "3x3_256_256@14": 13065212,   # algorithmic 8617984
+    "1x1_64_256@56": 109593638,   # algorithmic 109199360
+    "3x3_512_512@7": 23290891,    # algorithmic 6373376
+}
 
 
 def main():
@@ -34,6 +42,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / bit-exactness leg")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches only (no HIP graph replay)")
+    ap.add_argument("--profile", default=None, metavar="WHAT",
+                    help="launch one kernel 20 times and exit (for rocprofv3): a ResNet-50 layer name such as "
+                         "3x3_256_256@14, or gemm_i8 / gemm_f16 / copy")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus must be 1 "
@@ -69,9 +80,31 @@ def main():
         torch.cuda.synchronize()
         return s.elapsed_time(e) * 1e3 / iters
 
+    if args.profile in ("gemm_i8", "gemm_f16", "copy"):
+        n = 4096
+        if args.profile == "gemm_i8":
+            a = dev_t(rng.uniform_u8((n, n), 11))
+            w = dev_t(rng.uniform_s8((n, n), 12))
+            fn = lambda: U.dense(a, w)
+        elif args.profile == "gemm_f16":
+            a = dev_t(rng.normal_f16((n, n), 13, 1.0 / 64))
+            b = dev_t(rng.normal_f16((n, n), 14))
+            fn = lambda: U.gemm_fp16(a, b)
+        else:  # plain 128 MiB device-to-device copy: the calibration point for FETCH_SIZE / WRITE_SIZE
+            a = torch.empty(128 * 1024 * 1024, dtype=torch.uint8, device=dev)
+            b = torch.empty_like(a)
+            fn = lambda: b.copy_(a)
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
+        print(json.dumps({"profiled": args.profile, "launches": 20}))
+        return
+
     # ------------------------------------------------------------------ ResNet-50 b32 int8 conv stack
     layers = []
     for idx, s in enumerate(WL.RESNET50):
+        if args.profile and s.name != args.profile:
+            continue
         cb = WL.channel_block(s.C)
         cp = -(-s.C // cb) * cb
         data_np = rng.uniform_u8((BATCH, cp // cb, s.H, s.W, cb), 1000 + idx)
@@ -92,6 +125,15 @@ def main():
                            variant=U.last_variant(), ops=2 * WL.macs(s, BATCH),
                            bytes=WL.algorithmic_bytes(s, BATCH)))
     torch.cuda.synchronize()
+    if args.profile:
+        if not layers:
+            print(f"bench.py: unknown --profile target {args.profile!r}", file=sys.stderr)
+            sys.exit(2)
+        for _ in range(19):
+            layers[0]["call"]()
+        torch.cuda.synchronize()
+        print(json.dumps({"profiled": args.profile, "launches": 20, "kernel": layers[0]["variant"]}))
+        return
 
     def step():
         for ly in layers:
@@ -262,6 +304,12 @@ def main():
     layout["prepack_conv_weight_512x512x3x3"] = dict(us=round(us, 2), gbs=round(2 * w33.numel() / us / 1e3, 1))
     us = time_us(lambda: U.prepack_dense_weight(w8), 20)
     layout["prepack_dense_weight_4096x4096"] = dict(us=round(us, 2), gbs=round(2 * w8.numel() / us / 1e3, 1))
+    # plain device-to-device copy of known size: the HBM calibration point for the counters
+    src = torch.empty(128 * 1024 * 1024, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    us = time_us(lambda: dst.copy_(src), 10)
+    layout["plain_copy_128MiB"] = dict(us=round(us, 2), gbs=round(2 * src.numel() / us / 1e3, 1))
+    del src, dst
 
     # register-only MFMA throughput of this box (no memory traffic): what the silicon sustains
     sink = torch.zeros(4, dtype=torch.int32, device=dev)
@@ -272,12 +320,8 @@ def main():
         us = time_us(lambda: _lib.check(L.unit_mfma_peak(f16, blocks, iters, sink.data_ptr(), stream)), 3, warm=1)
         probe[key] = round(blocks * 16 * iters * per / us / 1e6, 1)
 
-    # HBM traffic of the dominant kernel, when a counter run has been recorded for it
-    try:
-        traffic = json.load(open(os.path.join(ROOT, "profiles", "traffic.json")))
-        roofline["traffic"] = traffic.get(roofline["layer"])
-    except (OSError, ValueError):
-        pass
+    # HBM traffic of the dominant kernel, when a counter run has been recorded for that layer
+    roofline["traffic"] = MEASURED_HBM_BYTES.get(roofline["layer"])
 
     # ------------------------------------------------------------------ CPU baseline + bit-exactness
     cpu_baseline = None
