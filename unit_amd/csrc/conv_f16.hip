@@ -25,13 +25,16 @@ int run_conv_f16(const unit_conv_desc *d, const ConvGeom &g0, const void *a, con
   typename YL::Params yp{static_cast<const char *>(a), g};
   typename Epi::Params ep{out, d->K, g.OH * g.OW, g.npix};
   const int gx = ceil_div(d->K, T::BX), gy = ceil_div(g.npix, T::BY);
-  set_variant("f16conv_x%d_y%d_k%d_w%d_p%d", T::BX, T::BY, T::BKB, T::NT / 64, PF);
+  set_variant("f16conv_x%d_y%d_k%d_w%d_p%d%s", T::BX, T::BY, T::BKB, T::NT / 64, PF, T::FF ? "f" : "");
   return launch_mma<OpF16, T, XL, YL, Epi, WS_NONE>(xp, yp, ep, nk, gx, gy, gx, 1, out, 0, g.ntab * 8, s,
                                                     "unit_conv2d_nchw16c_f16f32");
 }
 
 int run_conv_f16_variant(int variant, const unit_conv_desc *d, const ConvGeom &g, const void *a, const void *b,
                          void *out, hipStream_t s) {
+#define UNIT_CASE_FF(ID, BX, BY, BKB, WX, WY, PF) \
+  case ID:                                        \
+    return run_conv_f16<Tile<BX, BY, BKB, WX, WY, true>, PF>(d, g, a, b, out, s)
 #define UNIT_CASE(ID, BX, BY, BKB, WX, WY, PF) \
   case ID:                                     \
     return run_conv_f16<Tile<BX, BY, BKB, WX, WY>, PF>(d, g, a, b, out, s)
@@ -62,10 +65,25 @@ int run_conv_f16_variant(int variant, const unit_conv_desc *d, const ConvGeom &g
     UNIT_CASE(23, 128, 64, 128, 2, 2, 2);
     UNIT_CASE(24, 128, 128, 64, 2, 2, 3);
     UNIT_CASE(25, 256, 128, 64, 2, 2, 2);
+    UNIT_CASE(26, 64, 32, 128, 2, 1, 2);
+    UNIT_CASE(27, 128, 32, 128, 2, 1, 2);
+    UNIT_CASE(28, 64, 64, 128, 2, 1, 2);
+    UNIT_CASE(29, 64, 32, 64, 2, 1, 3);
+    UNIT_CASE(30, 128, 64, 128, 2, 1, 2);
+    UNIT_CASE(31, 128, 64, 128, 4, 1, 2);
+    UNIT_CASE_FF(32, 128, 64, 128, 2, 2, 2);
+    UNIT_CASE_FF(33, 64, 64, 64, 2, 2, 4);
+    UNIT_CASE_FF(34, 64, 32, 128, 2, 1, 2);
+    UNIT_CASE_FF(35, 128, 128, 128, 2, 2, 2);
+    UNIT_CASE_FF(36, 64, 128, 128, 1, 4, 2);
+    UNIT_CASE_FF(37, 128, 32, 128, 2, 1, 2);
+    UNIT_CASE_FF(38, 64, 64, 128, 2, 2, 2);
+    UNIT_CASE_FF(39, 128, 64, 128, 2, 2, 4);
     default:
       return fail(UNIT_E_ARG, "unit_conv2d_nchw16c_f16f32: unknown kernel variant %d", variant);
   }
 #undef UNIT_CASE
+#undef UNIT_CASE_FF
 }
 
 // measured on MI355X by `python -m unit_amd.tune --dtype f16` (key: N*OH*OW, K, C, KH, KW, stride)

@@ -10,6 +10,7 @@ namespace unit {
 
 struct TileShape {
   int bx, by, bkb, waves, pf;  // pf: stages of global loads in flight
+  bool ff = false;             // all fragments of a stage read at once (small wave tiles)
 };
 
 // index = variant id used by the tuning table and UNIT_AMD_CONV_VARIANT (1-based there)
@@ -40,6 +41,20 @@ constexpr TileShape kConvTiles[] = {
     {128, 64, 128, 4, 2},   // 23
     {128, 128, 64, 4, 3},   // 24
     {256, 128, 64, 4, 2},   // 25
+    {64, 32, 128, 2, 2},   // 26
+    {128, 32, 128, 2, 2},   // 27
+    {64, 64, 128, 2, 2},   // 28
+    {64, 32, 64, 2, 3},   // 29
+    {128, 64, 128, 2, 2},   // 30
+    {128, 64, 128, 4, 2},   // 31
+    {128, 64, 128, 4, 2, true},   // 32
+    {64, 64, 64, 4, 4, true},   // 33
+    {64, 32, 128, 2, 2, true},   // 34
+    {128, 128, 128, 4, 2, true},   // 35
+    {64, 128, 128, 4, 2, true},   // 36
+    {128, 32, 128, 2, 2, true},   // 37
+    {64, 64, 128, 4, 2, true},   // 38
+    {128, 64, 128, 4, 4, true},   // 39
 };
 constexpr int kNumConvTiles = sizeof(kConvTiles) / sizeof(kConvTiles[0]);
 

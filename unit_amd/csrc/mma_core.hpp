@@ -70,9 +70,13 @@ __device__ __forceinline__ int lds_off(int row, int chunk) {
   return row * BKB + ((chunk ^ swz<BKB>(row)) << 4);
 }
 
-template <int BX_, int BY_, int BKB_, int WX_, int WY_>
+// FF ("full fragments"): read the fragments of all k-steps of a stage at once, double-buffered per
+// stage, so a stage costs one LDS round trip instead of one per k-step.  For small wave tiles,
+// whose k-steps hold too few MFMAs to cover the LDS latency.
+template <int BX_, int BY_, int BKB_, int WX_, int WY_, bool FF_ = false>
 struct Tile {
   static constexpr int BX = BX_, BY = BY_, BKB = BKB_, WX = WX_, WY = WY_;
+  static constexpr bool FF = FF_;
   static constexpr int NT = WX * WY * 64;
   static constexpr int TX = BX / WX / 32, TY = BY / WY / 32;
   static constexpr int CPR = BKB / 16;           // 16-byte chunks per LDS row
@@ -159,7 +163,8 @@ __global__ __launch_bounds__(T::NT) void mma_kernel(typename XL::Params xp, type
   const int xsw = swz<T::BKB>(xrow), ysw = swz<T::BKB>(yrow);
   const int xbase = xrow * T::BKB, ybase = T::XBYTES + yrow * T::BKB;
 
-  v4i xf[2][T::TX], yf[2][T::TY];
+  constexpr int NSLOT = T::FF ? 2 * KK : 2;  // fragment register sets
+  v4i xf[NSLOT][T::TX], yf[NSLOT][T::TY];
   auto load_frags = [&](const char *stage, int kk, int slot) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < T::TX; ++i)
@@ -193,8 +198,9 @@ __global__ __launch_bounds__(T::NT) void mma_kernel(typename XL::Params xp, type
   // it into the slot just freed).
   constexpr int PF = XL::kPF;
   static_assert(XL::kPF == YL::kPF, "both operands use the same prefetch depth");
-  auto stage = [&](int kt, int par, auto slot, bool next, bool nextpf) __attribute__((always_inline)) {
+  auto stage = [&](int kt, int par, auto slot, auto fset, bool next, bool nextpf) __attribute__((always_inline)) {
     constexpr int U = decltype(slot)::value;
+    constexpr int FS = decltype(fset)::value;  // FF: fragment set that holds stage kt
     char *cur = lds + par * T::STAGE;
     char *nxt = lds + (par ^ 1) * T::STAGE;
     if (next) {
@@ -205,17 +211,30 @@ __global__ __launch_bounds__(T::NT) void mma_kernel(typename XL::Params xp, type
       xl.template fetch<U>(kt + 1 + PF);
       yl.template fetch<U>(kt + 1 + PF);
     }
+    if constexpr (T::FF) {
+      // all fragments of `cur` were requested one stage ago; after the barrier (which also
+      // waits for them) request all of `nxt`, then run the whole stage's MFMAs under those reads
+      __builtin_amdgcn_sched_barrier(0);
+      __syncthreads();
+      if (next) {
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-      if (kk + 1 < KK) {
-        load_frags(cur, kk + 1, (kk + 1) & 1);
-        mma_step(kk & 1);
-      } else {
-        __builtin_amdgcn_sched_barrier(0);
-        __syncthreads();  // everyone has read `cur` and written `nxt`
-        if (next) load_frags(nxt, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        mma_step(kk & 1);
+        for (int kk = 0; kk < KK; ++kk) load_frags(nxt, kk, (FS ^ 1) * KK + kk);
+      }
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) mma_step(FS * KK + kk);
+    } else {
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        if (kk + 1 < KK) {
+          load_frags(cur, kk + 1, (kk + 1) & 1);
+          mma_step(kk & 1);
+        } else {
+          __builtin_amdgcn_sched_barrier(0);
+          __syncthreads();  // everyone has read `cur` and written `nxt`
+          if (next) load_frags(nxt, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          mma_step(kk & 1);
+        }
       }
     }
   };
@@ -225,9 +244,12 @@ __global__ __launch_bounds__(T::NT) void mma_kernel(typename XL::Params xp, type
       constexpr int UU = decltype(u)::value;
       const int k = kt + UU;
       if constexpr (decltype(steady)::value) {
-        stage(k, (par + UU) & 1, std::integral_constant<int, (UU + 1) % PF>{}, true, true);
+        stage(k, (par + UU) & 1, std::integral_constant<int, (UU + 1) % PF>{}, std::integral_constant<int, UU & 1>{}, true,
+              true);
       } else {
-        if (k < ke) stage(k, (par + UU) & 1, std::integral_constant<int, (UU + 1) % PF>{}, k + 1 < ke, k + 1 + PF < ke);
+        if (k < ke)
+          stage(k, (par + UU) & 1, std::integral_constant<int, (UU + 1) % PF>{}, std::integral_constant<int, UU & 1>{},
+                k + 1 < ke, k + 1 + PF < ke);
       }
     };
     one(std::integral_constant<int, 0>{});
@@ -236,6 +258,7 @@ __global__ __launch_bounds__(T::NT) void mma_kernel(typename XL::Params xp, type
     if constexpr (PF > 3) one(std::integral_constant<int, 3>{});
   };
   static_assert(PF >= 1 && PF <= 4, "prefetch depth 1..4");
+  static_assert(!T::FF || PF % 2 == 0, "full-fragment mode alternates two fragment sets: even prefetch depth");
 
   if (XL::kNeedsSync || YL::kNeedsSync) __syncthreads();  // tap tables visible
   if (kb < ke) {
@@ -258,7 +281,12 @@ __global__ __launch_bounds__(T::NT) void mma_kernel(typename XL::Params xp, type
       yl.template fetch<0>(kb + PF);
     }
     __syncthreads();
-    load_frags(lds, 0, 0);
+    if constexpr (T::FF) {
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) load_frags(lds, kk, kk);
+    } else {
+      load_frags(lds, 0, 0);
+    }
     int kt = kb, par = 0;
     // steady state: every stage of the group has a successor and a stage PF+1 ahead to fetch
     for (; kt + 2 * PF < ke; kt += PF, par = (par + PF) & 1) stages_pf(kt, par, std::true_type{});

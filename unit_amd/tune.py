@@ -16,7 +16,7 @@ import json
 import os
 import sys
 
-NUM_VARIANTS = 26  # kConvTiles in csrc/conv_plan.hpp
+NUM_VARIANTS = 40  # kConvTiles in csrc/conv_plan.hpp
 
 
 def _shapes(spec):
@@ -44,13 +44,16 @@ def tune(spec, iters=20, verbose=True, dtype="i8"):
         for _ in range(3):
             fn()
         torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(iters):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1e3 / iters
+        best = float("inf")
+        for _ in range(3):  # best of three bursts: one burst next to a clock ramp misleads the choice
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(iters):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            best = min(best, e0.elapsed_time(e1) * 1e3 / iters)
+        return best
 
     saved = {k: os.environ.get(k) for k in ("UNIT_AMD_CONV_VARIANT", "UNIT_AMD_CONV_SPLITK")}
     results = []
