@@ -42,6 +42,10 @@ const char *unit_last_error(void);
  * (e.g. "i8conv_x256_y256_k128_w8"): the analogue of the tuned-schedule index the reference
  * logs per shape (python/tensorizer/tune.py:20-31). */
 const char *unit_last_variant(void);
+/* Number of tile variants the convolution entry points hold; the environment variable
+ * UNIT_AMD_CONV_VARIANT=1..count pins one per process, as the reference pins a schedule index
+ * through the tensorizer.tune globals (python/tensorizer/tune.py:3-16). */
+int unit_conv_variant_count(void);
 
 /* Geometry of one 2-D convolution; C and K are the channel counts as stored in the blocked
  * tensors (already rounded up: C % cb == 0, K % 16 == 0, apps/cpu/kernel/conv2d.py:18-22). */

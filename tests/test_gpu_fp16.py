@@ -83,6 +83,30 @@ def test_conv2d_fp16(dev, oracle, N, C, H, W, K, ks, stride):
     assert err <= REL_TOL, (err, U.last_variant())
 
 
+@pytest.mark.parametrize("N,C,H,W,K,ks,stride", [(2, 80, 9, 11, 96, 3, 1), (1, 32, 5, 5, 16, 1, 1), (3, 256, 9, 9, 160, 3, 2)])
+def test_conv2d_fp16_every_variant(dev, oracle, monkeypatch, N, C, H, W, K, ks, stride):
+    """Every tile variant gives the same result; integer-valued data makes fp32 accumulation exact
+    in any summation order, so the comparison with the float64 reference is bit for bit."""
+    from unit_amd import _lib
+    a = (rng.uniform_u8((N, C // 16, H, W, 16), 3 + C) % 7).astype(np.float16) - 3
+    b = (rng.uniform_u8((K // 16, C // 16, ks, ks, 16, 16), 4 + K) % 5).astype(np.float16) - 2
+    ref = oracle.conv2d_nchw16c_f16(a, b, stride, stride)
+    ta, tb = _t(a, dev), _t(b, dev)
+    count = _lib.load().unit_conv_variant_count()
+    ran = set()
+    for v in range(1, count + 1):
+        monkeypatch.setenv("UNIT_AMD_CONV_VARIANT", str(v))
+        try:
+            out = U.conv2d_NCHW16c_OHWI16o(ta, tb, stride, stride, "float32")
+        except ValueError as e:  # a variant may only be refused for its LDS budget or its layout
+            assert "LDS" in str(e) or "not available" in str(e), (v, str(e))
+            continue
+        torch.cuda.synchronize()
+        ran.add((v, U.last_variant()))
+        assert np.array_equal(out.cpu().numpy().astype(np.float64), ref), (v, U.last_variant())
+    assert len({name for _, name in ran}) == len({v for v, _ in ran}) >= 46
+
+
 def test_conv2d_fp16_unpacked_operands(dev, oracle):
     """4-D NCHW + OIHW operands are packed in-op like python/tensorizer/ops/gpu.py:25-33; integer
     data makes the comparison exact."""

@@ -102,6 +102,44 @@ def test_conv2d_bit_exact(dev, oracle, N, C, H, W, K, ks, stride, pad, dil):
     assert np.array_equal(out.cpu().numpy(), ref), U.last_variant()
 
 
+VARIANT_CASES = [
+    # N, C, H, W, K, kernel, stride, pad: reductions of 1 .. 12 pipeline stages, ragged tiles
+    (2, 80, 9, 11, 96, 3, 1, 1),    # 720 reduction bytes: the last stage is partly padding
+    (1, 32, 5, 5, 16, 1, 1, 0),     # one stage: k-groups beyond the first have nothing to do
+    (1, 48, 6, 6, 32, 3, 1, 1),     # 432 bytes: 4 or 7 stages, shared unevenly by 2 or 4 k-groups
+    (3, 256, 7, 7, 160, 3, 2, 1),   # 2304 bytes: a long reduction over few pixels
+    (1, 4, 16, 16, 32, 7, 2, 3),    # NCHW4c
+]
+
+
+@pytest.mark.parametrize("N,C,H,W,K,ks,stride,pad", VARIANT_CASES)
+def test_conv2d_every_variant(dev, oracle, monkeypatch, N, C, H, W, K, ks, stride, pad):
+    """Every tile variant the planner can pick (and k-splits of it) gives the oracle's result."""
+    from unit_amd import _lib
+    cb = 16 if C % 16 == 0 else 4
+    data = rng.uniform_u8((N, C // cb, H, W, cb), 11 * C + H)
+    wt = rng.uniform_s8((K // 16, C // cb, ks, ks, cb // 4, 16, 4), 5 * K + ks)
+    ref = oracle.c_conv2d_nchwc(data, wt, stride, pad, 1)
+    d, w = _t(data, dev), _t(wt, dev)
+    count = _lib.load().unit_conv_variant_count()
+    assert count >= 40
+    ran = set()
+    for v in range(1, count + 1):
+        for splits in (1, 3):
+            monkeypatch.setenv("UNIT_AMD_CONV_VARIANT", str(v))
+            monkeypatch.setenv("UNIT_AMD_CONV_SPLITK", str(splits))
+            try:
+                out = U.conv2d_NCHWc_int8(d, w, stride, pad, 1, "int32", f"NCHW{cb}c", "NCHW16c")
+            except ValueError as e:  # a variant may only be refused for its LDS budget or its layout
+                assert "LDS" in str(e) or "not available" in str(e), (v, str(e))
+                continue
+            torch.cuda.synchronize()
+            ran.add((v, U.last_variant()))
+            assert np.array_equal(out.cpu().numpy(), ref), (v, U.last_variant())
+    # the override really switched kernels: as many kernel names as variants that ran
+    assert len({name for _, name in ran}) >= len({v for v, _ in ran}) >= 46
+
+
 def test_conv2d_zero_padding_value(dev, oracle):
     """Padded pixels are u8 zeros: with all-255 data and all-ones weights every output equals
     255 * (number of in-image taps) * C, which differs between border and interior."""

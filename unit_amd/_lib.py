@@ -14,6 +14,7 @@ SYMBOLS = (
     "unit_version",
     "unit_last_error",
     "unit_last_variant",
+    "unit_conv_variant_count",
     "unit_conv_out_hw",
     "unit_conv2d_nchwc_u8s8s32",
     "unit_dense_dotprod_u8s8s32",

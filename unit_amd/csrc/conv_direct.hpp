@@ -1,0 +1,269 @@
+// int8 NCHW16c convolution with both MFMA operands read straight from global memory into
+// registers: no operand staging in LDS, no barrier in the reduction loop.
+//
+// Why: staging costs an LDS write and (wave tile permitting) several LDS reads per operand byte,
+// all through one 64-byte-per-clock pipe, and that pipe -- not the matrix cores -- bounds the
+// staged kernel whenever the output tile is small.  The layouts the reference uses happen to be
+// MFMA fragments already:
+//   * data (N, C/16, H, W, 16) u8: the 16 channels of one pixel and tap are 16 contiguous bytes
+//     = one lane's share of a k-step; consecutive lanes hold consecutive pixels (coalesced);
+//   * weights (K/16, C/16, KH, KW, 4, 16, 4) s8: for one tap, channel kb of a 16-channel block owns
+//     dwords at kb*4 + e*64, e = 0..3: four dword loads per lane, 64-byte runs per 16 lanes.
+// One k-step (32 reduction bytes per row) = two taps: lanes 0-31 hold tap 2s, lanes 32-63 tap 2s+1.
+//
+// A workgroup is KG waves that all compute the same (32 TX channels) x (32 TY pixels) tile, each
+// over its own share of the k-steps with a D-deep register prefetch ring; the partial tiles are
+// summed in LDS (integer adds: exact in any order) and the waves share the write-back.
+#pragma once
+#include "epilogues.hpp"
+#include "loaders.hpp"
+
+namespace unit {
+
+template <int TX_, int TY_, int KG_, int D_>
+struct DirectShape {
+  static constexpr int TX = TX_, TY = TY_, KG = KG_, D = D_;
+  static constexpr int BX = TX * 32, BY = TY * 32;
+  static constexpr int NT = 64 * KG;
+  static constexpr int kScratch = ConvEpilogue<OpI8>::kScratch;  // per-wave transpose area
+  static constexpr int SUM = TX * TY * 4096;                     // summed tile (KG > 1)
+  static constexpr int WSUM = TX * 32 * 4;                       // summed 128 * weight sums
+  static constexpr int LDS_FIXED = KG * kScratch + SUM + WSUM;   // the tap table follows
+  static_assert(NT <= 1024 && D >= 2 && D <= 8, "direct conv shape");
+};
+
+// Write one 32-channel x 32-pixel accumulator block (plus the per-channel correction in
+// wsb[32], LDS) to the (N, K/16, OH, OW, 16) output: transposed through the wave's LDS scratch so
+// that 64 lanes store 16 pixels x 64 bytes = 1 KiB of consecutive output per instruction.
+__device__ __forceinline__ void store_block_i8(const ConvEpilogue<OpI8>::Params &p, const v16i &acc, const int *wsb,
+                                               int c0, int m0, int lane, char *scratch) {
+  constexpr int kPitch = ConvEpilogue<OpI8>::kPitch;
+  const int l32 = lane & 31, half = lane >> 5;
+  const int rp = lane >> 2, piece = lane & 3;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    v4i v = {acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]};
+    v += *reinterpret_cast<const v4i *>(wsb + 8 * q + 4 * half);
+    *reinterpret_cast<v4i *>(scratch + l32 * kPitch + (8 * q + 4 * half) * 4) = v;
+  }
+  const int ko_planes = p.K >> 4;
+#pragma unroll
+  for (int it = 0; it < 2; ++it) {
+    const int m = m0 + it * 16 + rp;
+    const int n = m / p.ohw, pix = m - n * p.ohw;
+    const size_t obase = ((size_t)n * ko_planes * p.ohw + pix) * 16 + piece * 4;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int c = c0 + h * 16;
+      const v4i v = *reinterpret_cast<const v4i *>(scratch + (it * 16 + rp) * kPitch + h * 64 + piece * 16);
+      if (c < p.K && m < p.npix)
+        *reinterpret_cast<v4i *>(reinterpret_cast<int *>(p.out) + obase + (size_t)(c >> 4) * p.ohw * 16) = v;
+    }
+  }
+}
+
+template <class S>
+__global__ __launch_bounds__(S::NT) void conv_direct_i8(const char *__restrict__ data, const char *__restrict__ wgt,
+                                                        ConvEpilogue<OpI8>::Params ep, ConvGeom g, GridMap gm) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  constexpr int TX = S::TX, TY = S::TY, KG = S::KG, D = S::D;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int l32 = lane & 31, half = lane >> 5;
+
+  char *scratch = lds + wave * S::kScratch;
+  int *sum = reinterpret_cast<int *>(lds + KG * S::kScratch);
+  int *wsum = reinterpret_cast<int *>(lds + KG * S::kScratch + S::SUM);
+  v2i *tab = reinterpret_cast<v2i *>(lds + S::LDS_FIXED);
+
+  // tap -> (byte offset of the tap inside an image relative to the window origin, window bit);
+  // the odd tap past the end gets bit 0: it is staged like zero padding
+  const int nsteps = (g.ntaps + 1) >> 1;
+  for (int e = threadIdx.x; e < 2 * nsteps; e += S::NT) {
+    v2i ent = {0, 0};
+    if (e < g.ntaps) {
+      const int kw = e % g.KW, rest = e / g.KW, kh = rest % g.KH, ci = rest / g.KH;
+      ent[0] = ((ci * g.H + kh * g.dh) * g.W + kw * g.dw) * 16;
+      ent[1] = (int)(1u << (kh * g.KW + kw));
+    }
+    tab[e] = ent;
+  }
+  if constexpr (KG > 1) {
+    for (int e = threadIdx.x; e < (S::SUM + S::WSUM) / 4; e += S::NT) sum[e] = 0;
+  }
+
+  int bx, by, split;
+  gm.locate(blockIdx.x, bx, by, split);
+  const int x0 = bx * S::BX, y0 = by * S::BY;
+
+  // weights: byte offset of this lane's channel at tap 0, per 32-channel block (rows past K
+  // re-read the last channel; their results are never stored)
+  u32 xoff[TX];
+#pragma unroll
+  for (int i = 0; i < TX; ++i) {
+    int n = x0 + i * 32 + l32;
+    n = n < ep.K ? n : ep.K - 1;
+    xoff[i] = (u32)(n >> 4) * (u32)(g.ntaps * 256) + (u32)(n & 15) * 4u;
+  }
+  // data: byte offset of the window origin of this lane's pixel per 32-pixel block, and the set of
+  // window positions (kh, kw) that fall inside the image (none for lanes past the last pixel)
+  int pixoff[TY];
+  u32 inside[TY];
+#pragma unroll
+  for (int j = 0; j < TY; ++j) {
+    const int m = y0 + j * 32 + l32;
+    pixoff[j] = 0;
+    inside[j] = 0;
+    if (m < g.npix) {
+      const int n = m / (g.OH * g.OW), rem = m - n * (g.OH * g.OW);
+      const int oh = rem / g.OW, ow = rem - oh * g.OW;
+      const int ih0 = oh * g.sh - g.pt, iw0 = ow * g.sw - g.pl;
+      pixoff[j] = (int)(n * g.img_bytes) + (ih0 * g.W + iw0) * 16;
+      u32 bits = 0;
+      for (int kh = 0; kh < g.KH; ++kh)
+        for (int kw = 0; kw < g.KW; ++kw)
+          if ((u32)(ih0 + kh * g.dh) < (u32)g.H && (u32)(iw0 + kw * g.dw) < (u32)g.W) bits |= 1u << (kh * g.KW + kw);
+      inside[j] = bits;
+    }
+  }
+
+  typename OpI8::acc_t acc[TX][TY];
+#pragma unroll
+  for (int i = 0; i < TX; ++i)
+#pragma unroll
+    for (int j = 0; j < TY; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+  int wsx[TX];
+#pragma unroll
+  for (int i = 0; i < TX; ++i) wsx[i] = 0;
+
+  // prefetch ring: D k-steps of fragments in registers
+  v4i xf[D][TX], yf[D][TY];
+  int ym[D][TY];  // all ones where the tap lies inside the image, else 0
+  const u32 last_tap_off = (u32)(g.ntaps - 1) * 256u;
+
+  auto fetch = [&](auto slot, int s) __attribute__((always_inline)) {
+    constexpr int U = decltype(slot)::value;
+    const int t = 2 * s + half;
+    const v2i e = tab[t];
+    // the odd tap past the end re-reads the last tap's weights: its data is staged as zero
+    // padding, and a padded position contributes -128 * w to the accumulator and +128 * w through
+    // the weight-sum correction, whatever w is
+    u32 xk = (u32)t * 256u;
+    xk = xk < last_tap_off ? xk : last_tap_off;
+#pragma unroll
+    for (int i = 0; i < TX; ++i) {
+      const char *p = wgt + xoff[i] + xk;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) xf[U][i][d] = *reinterpret_cast<const int *>(p + d * 64);
+    }
+#pragma unroll
+    for (int j = 0; j < TY; ++j) {
+      const bool ok = (inside[j] & (u32)e[1]) != 0;
+      yf[U][j] = *reinterpret_cast<const v4i *>(data + (ok ? pixoff[j] + e[0] : 0));
+      ym[U][j] = ok ? -1 : 0;
+    }
+  };
+  auto consume = [&](auto slot) __attribute__((always_inline)) {
+    constexpr int U = decltype(slot)::value;
+    v4i y[TY];
+#pragma unroll
+    for (int j = 0; j < TY; ++j)
+#pragma unroll
+      for (int d = 0; d < 4; ++d) y[j][d] = (yf[U][j][d] & ym[U][j]) ^ (int)0x80808080;
+#pragma unroll
+    for (int i = 0; i < TX; ++i)
+#pragma unroll
+      for (int d = 0; d < 4; ++d) wsx[i] = __builtin_amdgcn_sdot4(xf[U][i][d], 0x01010101, wsx[i], false);
+#pragma unroll
+    for (int i = 0; i < TX; ++i)
+#pragma unroll
+      for (int j = 0; j < TY; ++j) acc[i][j] = OpI8::mma(xf[U][i], y[j], acc[i][j]);
+  };
+  // D consecutive k-steps starting at s, slots resolved at compile time
+  auto ring = [&](int s, int s1, auto steady) __attribute__((always_inline)) {
+    auto one = [&](auto u) __attribute__((always_inline)) {
+      constexpr int UU = decltype(u)::value;
+      if constexpr (decltype(steady)::value) {
+        consume(u);
+        fetch(u, s + UU + D);
+      } else {
+        if (s + UU < s1) {
+          consume(u);
+          if (s + UU + D < s1) fetch(u, s + UU + D);
+        }
+      }
+    };
+    one(std::integral_constant<int, 0>{});
+    one(std::integral_constant<int, 1>{});
+    if constexpr (D > 2) one(std::integral_constant<int, 2>{});
+    if constexpr (D > 3) one(std::integral_constant<int, 3>{});
+    if constexpr (D > 4) one(std::integral_constant<int, 4>{});
+    if constexpr (D > 5) one(std::integral_constant<int, 5>{});
+    if constexpr (D > 6) one(std::integral_constant<int, 6>{});
+    if constexpr (D > 7) one(std::integral_constant<int, 7>{});
+  };
+
+  __syncthreads();  // tap table (and the zeroed sums) visible
+
+  const int s0 = nsteps * wave / KG, s1 = nsteps * (wave + 1) / KG;
+  {
+    auto pre = [&](auto u) __attribute__((always_inline)) {
+      constexpr int UU = decltype(u)::value;
+      if (s0 + UU < s1) fetch(u, s0 + UU);
+    };
+    pre(std::integral_constant<int, 0>{});
+    pre(std::integral_constant<int, 1>{});
+    if constexpr (D > 2) pre(std::integral_constant<int, 2>{});
+    if constexpr (D > 3) pre(std::integral_constant<int, 3>{});
+    if constexpr (D > 4) pre(std::integral_constant<int, 4>{});
+    if constexpr (D > 5) pre(std::integral_constant<int, 5>{});
+    if constexpr (D > 6) pre(std::integral_constant<int, 6>{});
+    if constexpr (D > 7) pre(std::integral_constant<int, 7>{});
+  }
+  int s = s0;
+  for (; s + 2 * D <= s1; s += D) ring(s, s1, std::true_type{});
+  for (; s < s1; s += D) ring(s, s1, std::false_type{});
+
+  // the two 32-lane halves hold the weight sums of the two taps of every k-step
+#pragma unroll
+  for (int i = 0; i < TX; ++i) wsx[i] = (wsx[i] + __shfl_xor(wsx[i], 32)) << 7;
+
+  if constexpr (KG == 1) {
+    if (half == 0) {
+#pragma unroll
+      for (int i = 0; i < TX; ++i) wsum[i * 32 + l32] = wsx[i];
+    }
+#pragma unroll
+    for (int i = 0; i < TX; ++i)
+#pragma unroll
+      for (int j = 0; j < TY; ++j)
+        store_block_i8(ep, acc[i][j], wsum + i * 32, x0 + i * 32, y0 + j * 32, lane, scratch);
+  } else {
+    // sum the partial tiles of the KG waves in LDS, then share the blocks among the waves
+#pragma unroll
+    for (int i = 0; i < TX; ++i)
+#pragma unroll
+      for (int j = 0; j < TY; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          __hip_atomic_fetch_add(sum + ((i * TY + j) * 16 + r) * 64 + lane, acc[i][j][r], __ATOMIC_RELAXED,
+                                 __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (half == 0) {
+#pragma unroll
+      for (int i = 0; i < TX; ++i)
+        __hip_atomic_fetch_add(wsum + i * 32 + l32, wsx[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    __syncthreads();
+    for (int b = wave; b < TX * TY; b += KG) {
+      const int i = b / TY, j = b - i * TY;
+      v16i total;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) total[r] = sum[(b * 16 + r) * 64 + lane];
+      store_block_i8(ep, total, wsum + i * 32, x0 + i * 32, y0 + j * 32, lane, scratch);
+    }
+  }
+}
+
+}  // namespace unit

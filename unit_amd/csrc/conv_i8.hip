@@ -4,19 +4,23 @@
 namespace unit {
 
 int conv_geom(const unit_conv_desc *d, int tapb, ConvGeom *g, const char *what);  // abi.hip
-int conv_i8_c16(int variant, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w, void *out,
-                int splits, hipStream_t s);
-int conv_i8_c4(int variant, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w, void *out,
-               int splits, hipStream_t s);
+int conv_i8_c16(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
+                void *out, hipStream_t s);
+int conv_i8_direct(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
+                   void *out, hipStream_t s);
+int conv_i8_c4(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
+               void *out, hipStream_t s);
 
 namespace {
 // measured on MI355X by `python -m unit_amd.tune` (key: N*OH*OW, K, C, KH, KW, stride)
 const TunedConv kTunedI8[] = {
 #include "tuned_conv_i8.inc"
-    {0, 0, 0, 0, 0, 0, 0, 0},
+    {0, 0, 0, 0, 0, 0, 0, 0, 0},
 };
 }  // namespace
 }  // namespace unit
+
+extern "C" int unit_conv_variant_count(void) { return unit::kNumConvTiles; }
 
 extern "C" int unit_conv2d_nchwc_u8s8s32(const unit_conv_desc *d, const void *data, const void *weight,
                                          void *out, unit_stream_t stream) {
@@ -31,6 +35,6 @@ extern "C" int unit_conv2d_nchwc_u8s8s32(const unit_conv_desc *d, const void *da
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int ntable = (int)(sizeof(kTunedI8) / sizeof(kTunedI8[0])) - 1;
   const ConvPlan p = plan_conv(d, g.npix, g.ntaps * d->cb, kTunedI8, ntable, true);
-  return d->cb == 16 ? conv_i8_c16(p.variant, d, g, data, weight, out, p.splits, s)
-                     : conv_i8_c4(p.variant, d, g, data, weight, out, p.splits, s);
+  if (kConvTiles[p.variant].direct) return conv_i8_direct(p, d, g, data, weight, out, s);
+  return d->cb == 16 ? conv_i8_c16(p, d, g, data, weight, out, s) : conv_i8_c4(p, d, g, data, weight, out, s);
 }

@@ -9,10 +9,10 @@
 namespace unit {
 
 template <class T, int TAPB, int PF>
-int run_conv_i8(const unit_conv_desc *d, const ConvGeom &g0, const void *data, const void *w, void *out, int splits,
-                hipStream_t s) {
-  using XL = VnniLoader<T::BX, T::BKB, T::NT, 16, PF>;
-  using YL = ConvPixelLoader<T::BY, T::BKB, T::NT, TAPB, true, PF>;
+int run_conv_i8(const unit_conv_desc *d, const ConvGeom &g0, const void *data, const void *w, void *out,
+                const ConvPlan &plan, hipStream_t s) {
+  using XL = VnniLoader<T::BX, T::BKB, T::NTG, 16, PF>;
+  using YL = ConvPixelLoader<T::BY, T::BKB, T::NTG, TAPB, true, PF>;
   using Epi = ConvEpilogue<OpI8>;
   ConvGeom g = g0;
   const int kbytes = g.ntaps * TAPB;
@@ -22,68 +22,31 @@ int run_conv_i8(const unit_conv_desc *d, const ConvGeom &g0, const void *data, c
   typename YL::Params yp{static_cast<const char *>(data), g};
   typename Epi::Params ep{out, d->K, g.OH * g.OW, g.npix};
   const int gx = ceil_div(d->K, T::BX), gy = ceil_div(g.npix, T::BY);
-  if (splits > nk) splits = nk;
-  set_variant("i8conv_c%d_x%d_y%d_k%d_w%d_p%d%s_s%d", TAPB, T::BX, T::BY, T::BKB, T::NT / 64, PF, T::FF ? "f" : "", splits);
-  return launch_mma<OpI8, T, XL, YL, Epi, WS_X>(xp, yp, ep, nk, gx, gy, gx, splits, out,
+  const int splits = plan.splits > nk ? nk : plan.splits;
+  const int panel = plan.panel > 0 && plan.panel < gx ? plan.panel : 0;
+  char tail[16] = "";
+  if (panel) snprintf(tail, sizeof tail, "_r%d", panel);
+  set_variant("i8conv_c%d_x%d_y%d_k%d_w%dx%d_p%d%s%s%s_s%d", TAPB, T::BX, T::BY, T::BKB, T::WX, T::WY, PF, T::FF ? "f" : "",
+              T::KG == 1 ? "" : (T::KG == 2 ? "_g2" : "_g4"), tail, splits);
+  return launch_mma<OpI8, T, XL, YL, Epi, WS_X>(xp, yp, ep, nk, gx, gy, panel ? panel : gx, splits, out,
                                                 (size_t)g.npix * d->K * 4, g.ntab * 8, s,
                                                 "unit_conv2d_nchwc_u8s8s32");
 }
 
 template <int TAPB>
-int run_conv_i8_variant(int variant, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
-                        void *out, int splits, hipStream_t s) {
-#define UNIT_CASE_FF(ID, BX, BY, BKB, WX, WY, PF) \
-  case ID:                                        \
-    return run_conv_i8<Tile<BX, BY, BKB, WX, WY, true>, TAPB, PF>(d, g, data, w, out, splits, s)
-#define UNIT_CASE(ID, BX, BY, BKB, WX, WY, PF) \
-  case ID:                                     \
-    return run_conv_i8<Tile<BX, BY, BKB, WX, WY>, TAPB, PF>(d, g, data, w, out, splits, s)
-  switch (variant) {
-    UNIT_CASE(0, 256, 256, 128, 2, 4, 1);
-    UNIT_CASE(1, 256, 256, 64, 2, 4, 1);
-    UNIT_CASE(2, 128, 256, 128, 2, 4, 1);
-    UNIT_CASE(3, 128, 256, 64, 2, 4, 1);
-    UNIT_CASE(4, 64, 256, 128, 1, 4, 1);
-    UNIT_CASE(5, 64, 256, 64, 1, 4, 1);
-    UNIT_CASE(6, 128, 128, 128, 2, 2, 1);
-    UNIT_CASE(7, 128, 128, 64, 2, 2, 1);
-    UNIT_CASE(8, 256, 128, 128, 2, 2, 1);
-    UNIT_CASE(9, 256, 128, 64, 2, 2, 1);
-    UNIT_CASE(10, 64, 128, 64, 1, 4, 1);
-    UNIT_CASE(11, 64, 64, 64, 2, 2, 1);
-    UNIT_CASE(12, 256, 256, 128, 2, 2, 1);
-    UNIT_CASE(13, 256, 256, 64, 2, 2, 1);
-    UNIT_CASE(14, 128, 64, 128, 2, 2, 1);
-    UNIT_CASE(15, 64, 128, 128, 1, 4, 1);
-    UNIT_CASE(16, 128, 64, 128, 2, 2, 3);
-    UNIT_CASE(17, 64, 128, 128, 1, 4, 3);
-    UNIT_CASE(18, 128, 128, 128, 2, 2, 2);
-    UNIT_CASE(19, 64, 64, 64, 2, 2, 4);
-    UNIT_CASE(20, 64, 256, 64, 1, 4, 2);
-    UNIT_CASE(21, 64, 128, 64, 1, 4, 3);
-    UNIT_CASE(22, 128, 256, 128, 2, 4, 2);
-    UNIT_CASE(23, 128, 64, 128, 2, 2, 2);
-    UNIT_CASE(24, 128, 128, 64, 2, 2, 3);
-    UNIT_CASE(25, 256, 128, 64, 2, 2, 2);
-    UNIT_CASE(26, 64, 32, 128, 2, 1, 2);
-    UNIT_CASE(27, 128, 32, 128, 2, 1, 2);
-    UNIT_CASE(28, 64, 64, 128, 2, 1, 2);
-    UNIT_CASE(29, 64, 32, 64, 2, 1, 3);
-    UNIT_CASE(30, 128, 64, 128, 2, 1, 2);
-    UNIT_CASE(31, 128, 64, 128, 4, 1, 2);
-    UNIT_CASE_FF(32, 128, 64, 128, 2, 2, 2);
-    UNIT_CASE_FF(33, 64, 64, 64, 2, 2, 4);
-    UNIT_CASE_FF(34, 64, 32, 128, 2, 1, 2);
-    UNIT_CASE_FF(35, 128, 128, 128, 2, 2, 2);
-    UNIT_CASE_FF(36, 64, 128, 128, 1, 4, 2);
-    UNIT_CASE_FF(37, 128, 32, 128, 2, 1, 2);
-    UNIT_CASE_FF(38, 64, 64, 128, 2, 2, 2);
-    UNIT_CASE_FF(39, 128, 64, 128, 2, 2, 4);
+int run_conv_i8_variant(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data,
+                        const void *w, void *out, hipStream_t s) {
+#define UNIT_CONV_DIRECT(ID, TX, TY, KG, D)
+#define UNIT_CONV_VARIANT(ID, BX, BY, BKB, WX, WY, PF, FF, KG) \
+  case ID:                                                     \
+    return run_conv_i8<Tile<BX, BY, BKB, WX, WY, FF, KG>, TAPB, PF>(d, g, data, w, out, plan, s);
+  switch (plan.variant) {
+#include "conv_variants.def"
     default:
-      return fail(UNIT_E_ARG, "unit_conv2d_nchwc_u8s8s32: unknown kernel variant %d", variant);
+      return fail(UNIT_E_ARG, "unit_conv2d_nchwc_u8s8s32: kernel variant %d not available for this layout", plan.variant);
   }
-#undef UNIT_CASE
-#undef UNIT_CASE_FF
+#undef UNIT_CONV_VARIANT
+#undef UNIT_CONV_DIRECT
 }
 
 }  // namespace unit

@@ -9,63 +9,35 @@
 namespace unit {
 
 struct TileShape {
-  int bx, by, bkb, waves, pf;  // pf: stages of global loads in flight
-  bool ff = false;             // all fragments of a stage read at once (small wave tiles)
+  int bx, by, bkb, waves, pf;  // waves per workgroup; pf: stages of global loads in flight
+  bool ff;                     // all fragments of a stage read at once (small wave tiles)
+  int kg;                      // k-groups sharing the output tile
+  bool direct;                 // operands straight from global memory to registers (int8 NCHW16c)
 };
 
 // index = variant id used by the tuning table and UNIT_AMD_CONV_VARIANT (1-based there)
 constexpr TileShape kConvTiles[] = {
-    {256, 256, 128, 8, 1},  // 0
-    {256, 256, 64, 8, 1},   // 1
-    {128, 256, 128, 8, 1},  // 2
-    {128, 256, 64, 8, 1},   // 3
-    {64, 256, 128, 4, 1},   // 4
-    {64, 256, 64, 4, 1},    // 5
-    {128, 128, 128, 4, 1},  // 6
-    {128, 128, 64, 4, 1},   // 7
-    {256, 128, 128, 4, 1},  // 8
-    {256, 128, 64, 4, 1},   // 9
-    {64, 128, 64, 4, 1},    // 10
-    {64, 64, 64, 4, 1},     // 11
-    {256, 256, 128, 4, 1},  // 12
-    {256, 256, 64, 4, 1},   // 13
-    {128, 64, 128, 4, 1},   // 14
-    {64, 128, 128, 4, 1},   // 15
-    {128, 64, 128, 4, 3},   // 16
-    {64, 128, 128, 4, 3},   // 17
-    {128, 128, 128, 4, 2},  // 18
-    {64, 64, 64, 4, 4},     // 19
-    {64, 256, 64, 4, 2},    // 20
-    {64, 128, 64, 4, 3},    // 21
-    {128, 256, 128, 8, 2},  // 22
-    {128, 64, 128, 4, 2},   // 23
-    {128, 128, 64, 4, 3},   // 24
-    {256, 128, 64, 4, 2},   // 25
-    {64, 32, 128, 2, 2},   // 26
-    {128, 32, 128, 2, 2},   // 27
-    {64, 64, 128, 2, 2},   // 28
-    {64, 32, 64, 2, 3},   // 29
-    {128, 64, 128, 2, 2},   // 30
-    {128, 64, 128, 4, 2},   // 31
-    {128, 64, 128, 4, 2, true},   // 32
-    {64, 64, 64, 4, 4, true},   // 33
-    {64, 32, 128, 2, 2, true},   // 34
-    {128, 128, 128, 4, 2, true},   // 35
-    {64, 128, 128, 4, 2, true},   // 36
-    {128, 32, 128, 2, 2, true},   // 37
-    {64, 64, 128, 4, 2, true},   // 38
-    {128, 64, 128, 4, 4, true},   // 39
+#define UNIT_CONV_VARIANT(ID, BX, BY, BKB, WX, WY, PF, FF, KG) {BX, BY, BKB, (WX) * (WY) * (KG), PF, FF, KG, false},
+#define UNIT_CONV_DIRECT(ID, TX, TY, KG, D) {(TX) * 32, (TY) * 32, 32, KG, D, false, KG, true},
+#include "conv_variants.def"
+#undef UNIT_CONV_DIRECT
+#undef UNIT_CONV_VARIANT
 };
 constexpr int kNumConvTiles = sizeof(kConvTiles) / sizeof(kConvTiles[0]);
 
 struct ConvPlan {
   int variant;
   int splits;
+  // Channel tiles per panel of the workgroup -> tile walk (0: all of them).  An XCD's workgroups
+  // cover whole panels, so 0 makes every XCD read all weights and a slice of the pixels, while
+  // a small panel gives each XCD a slice of the weights and all pixels: the better choice is the
+  // one that pulls fewer bytes into the 8 L2s, which start cold at every kernel.
+  int panel;
 };
 
 struct TunedConv {
   int npix, K, C, KH, KW, sh;  // key
-  int variant, splits;
+  int variant, splits, panel;
 };
 
 // Heuristic for shapes the table does not hold, distilled from the tuning runs: output-bound
@@ -96,22 +68,26 @@ inline ConvPlan heuristic_plan(int npix, int K, int kbytes, bool allow_split) {
     const int nk = ceil_div(kbytes, t.bkb);
     while (nt * splits < 96 && nk / (splits * 2) >= 4 && splits < 8) splits *= 2;
   }
-  return ConvPlan{v, splits};
+  return ConvPlan{v, splits, 0};
 }
 
 inline ConvPlan plan_conv(const unit_conv_desc *d, int npix, int kbytes, const TunedConv *table, int ntable,
                           bool allow_split) {
   ConvPlan p = heuristic_plan(npix, d->K, kbytes, allow_split);
+  // UNIT_AMD_CONV_NOTABLE=1: heuristic only (the tuner measures it as the baseline)
+  if (tuning_override("UNIT_AMD_CONV_NOTABLE") > 0) ntable = 0;
   for (int i = 0; i < ntable; ++i) {
     const TunedConv &e = table[i];
     if (e.npix == npix && e.K == d->K && e.C == d->C && e.KH == d->KH && e.KW == d->KW && e.sh == d->sh) {
-      p = ConvPlan{e.variant, e.splits};
+      p = ConvPlan{e.variant, e.splits, e.panel};
       break;
     }
   }
   const int ov = tuning_override("UNIT_AMD_CONV_VARIANT"), os = tuning_override("UNIT_AMD_CONV_SPLITK");
   if (ov > 0 && ov <= kNumConvTiles) p.variant = ov - 1;
   if (os > 0) p.splits = os;
+  const int op = tuning_override("UNIT_AMD_CONV_PANEL");
+  if (op > 0) p.panel = op;
   if (!allow_split) p.splits = 1;
   return p;
 }

@@ -74,7 +74,7 @@ struct ConvEpilogue {
   // LDS bytes the epilogue needs for a tile shape
   template <class T>
   static constexpr int lds_bytes() {
-    return (T::NT / 64) * (kScratch + T::TX * 32 * 4);
+    return (T::NTG / 64) * (kScratch + T::TX * 32 * 4);
   }
 
   template <class T>
@@ -85,7 +85,7 @@ struct ConvEpilogue {
     using out4_t = typename Op::out4_t;
     const int l32 = lane & 31, half = lane >> 5;
     char *scratch = lds + wave * kScratch;
-    int *wsb = reinterpret_cast<int *>(lds + (T::NT / 64) * kScratch) + wave * (T::TX * 32);
+    int *wsb = reinterpret_cast<int *>(lds + (T::NTG / 64) * kScratch) + wave * (T::TX * 32);
     if constexpr (Op::kInt) {
       if (half == 0) {
 #pragma unroll

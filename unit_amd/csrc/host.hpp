@@ -49,7 +49,7 @@ template <class Op, class T, class XL, class YL, class Epi, int WS>
 int launch_mma(const typename XL::Params &xp, const typename YL::Params &yp, const typename Epi::Params &ep,
                int nk, int gx, int gy, int ph, int splits, void *out, size_t out_bytes, int aux_bytes,
                hipStream_t stream, const char *what) {
-  constexpr int epi = Epi::template lds_bytes<T>();
+  constexpr int epi = Epi::template lds_bytes<T>() + T::XCHG;  // epilogue scratch + k-group hand-over
   const int lds = (T::LDS_TILES + aux_bytes) > epi ? (T::LDS_TILES + aux_bytes) : epi;
   if (lds > kMaxLds) return fail(UNIT_E_ARG, "%s: needs %d bytes of LDS (limit %d)", what, lds, kMaxLds);
   auto kern = mma_kernel<Op, T, XL, YL, Epi, WS>;

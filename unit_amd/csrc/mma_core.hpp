@@ -73,17 +73,26 @@ __device__ __forceinline__ int lds_off(int row, int chunk) {
 // FF ("full fragments"): read the fragments of all k-steps of a stage at once, double-buffered per
 // stage, so a stage costs one LDS round trip instead of one per k-step.  For small wave tiles,
 // whose k-steps hold too few MFMAs to cover the LDS latency.
-template <int BX_, int BY_, int BKB_, int WX_, int WY_, bool FF_ = false>
+//
+// KG ("k-groups"): KG sets of WX x WY waves work on the same output tile, each set on its own
+// share of the workgroup's reduction range with its own loaders and LDS buffers; their
+// accumulators are summed through LDS before the epilogue.  For layers with few output tiles and
+// a long reduction: KG times the loads in flight and KG waves per SIMD without device atomics.
+template <int BX_, int BY_, int BKB_, int WX_, int WY_, bool FF_ = false, int KG_ = 1>
 struct Tile {
-  static constexpr int BX = BX_, BY = BY_, BKB = BKB_, WX = WX_, WY = WY_;
+  static constexpr int BX = BX_, BY = BY_, BKB = BKB_, WX = WX_, WY = WY_, KG = KG_;
   static constexpr bool FF = FF_;
-  static constexpr int NT = WX * WY * 64;
+  static constexpr int NTG = WX * WY * 64;       // threads of one k-group
+  static constexpr int NT = NTG * KG;
   static constexpr int TX = BX / WX / 32, TY = BY / WY / 32;
   static constexpr int CPR = BKB / 16;           // 16-byte chunks per LDS row
   static constexpr int XBYTES = BX * BKB, YBYTES = BY * BKB;
   static constexpr int STAGE = XBYTES + YBYTES;
-  static constexpr int LDS_TILES = 2 * STAGE;
+  static constexpr int LDS_TILES = 2 * STAGE * KG;
+  // accumulators and weight sums of the k-groups other than the first, handed over through LDS
+  static constexpr int XCHG = (KG - 1) * (BX * BY * 4 + (NTG / 64) * (TX + TY) * 256);
   static_assert(BX % (WX * 32) == 0 && BY % (WY * 32) == 0, "wave tile is a multiple of 32x32");
+  static_assert(KG >= 1 && NT <= 1024, "at most 16 waves per workgroup");
 };
 
 // Workgroup id -> (tile, k-split).  Workgroups are dealt round-robin to the 8 XCDs, each with
@@ -124,8 +133,12 @@ template <class Op, class T, class XL, class YL, class Epi, int WS>
 __global__ __launch_bounds__(T::NT) void mma_kernel(typename XL::Params xp, typename YL::Params yp,
                                                     typename Epi::Params ep, int nk_total, GridMap gm) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  const int t = threadIdx.x;
-  const int lane = t & 63, wave = t >> 6;
+  const int lane = threadIdx.x & 63;
+  // k-group and wave inside it, as scalars: every branch below that depends on them is uniform
+  const int wave_wg = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int grp = T::KG > 1 ? wave_wg / (T::WX * T::WY) : 0;
+  const int wave = wave_wg - grp * (T::WX * T::WY);
+  const int t = wave * 64 + lane;  // thread id inside the k-group
   const int wx = wave % T::WX, wy = wave / T::WX;
   const int l32 = lane & 31, half = lane >> 5;
   constexpr int KK = T::BKB / 32;
@@ -134,8 +147,10 @@ __global__ __launch_bounds__(T::NT) void mma_kernel(typename XL::Params xp, type
   int bx, by, split;
   gm.locate(blockIdx.x, bx, by, split);
   const int x0 = bx * T::BX, y0 = by * T::BY;
-  // this workgroup's stages: [kb, ke)
-  const int kb = (int)((long)nk_total * split / gm.splits), ke = (int)((long)nk_total * (split + 1) / gm.splits);
+  // this workgroup's stages [kb0, ke0), this k-group's share of them [kb, ke)
+  const int kb0 = (int)((long)nk_total * split / gm.splits), ke0 = (int)((long)nk_total * (split + 1) / gm.splits);
+  const int kb = kb0 + (ke0 - kb0) * grp / T::KG, ke = kb0 + (ke0 - kb0) * (grp + 1) / T::KG;
+  char *const tiles = lds + grp * (2 * T::STAGE);  // this k-group's LDS double buffer
 
   XL xl;
   YL yl;
@@ -201,8 +216,8 @@ __global__ __launch_bounds__(T::NT) void mma_kernel(typename XL::Params xp, type
   auto stage = [&](int kt, int par, auto slot, auto fset, bool next, bool nextpf) __attribute__((always_inline)) {
     constexpr int U = decltype(slot)::value;
     constexpr int FS = decltype(fset)::value;  // FF: fragment set that holds stage kt
-    char *cur = lds + par * T::STAGE;
-    char *nxt = lds + (par ^ 1) * T::STAGE;
+    char *cur = tiles + par * T::STAGE;
+    char *nxt = tiles + (par ^ 1) * T::STAGE;
     if (next) {
       xl.template commit<U>(nxt);
       yl.template commit<U>(nxt + T::XBYTES);
@@ -274,8 +289,8 @@ __global__ __launch_bounds__(T::NT) void mma_kernel(typename XL::Params xp, type
     if constexpr (PF > 3) {
       if (kb + 3 < ke) { xl.template fetch<3 % PF>(kb + 3); yl.template fetch<3 % PF>(kb + 3); }
     }
-    xl.template commit<0>(lds);
-    yl.template commit<0>(lds + T::XBYTES);
+    xl.template commit<0>(tiles);
+    yl.template commit<0>(tiles + T::XBYTES);
     if (kb + PF < ke) {
       xl.template fetch<0>(kb + PF);
       yl.template fetch<0>(kb + PF);
@@ -283,9 +298,9 @@ __global__ __launch_bounds__(T::NT) void mma_kernel(typename XL::Params xp, type
     __syncthreads();
     if constexpr (T::FF) {
 #pragma unroll
-      for (int kk = 0; kk < KK; ++kk) load_frags(lds, kk, kk);
+      for (int kk = 0; kk < KK; ++kk) load_frags(tiles, kk, kk);
     } else {
-      load_frags(lds, 0, 0);
+      load_frags(tiles, 0, 0);
     }
     int kt = kb, par = 0;
     // steady state: every stage of the group has a successor and a stage PF+1 ahead to fetch
@@ -301,6 +316,55 @@ __global__ __launch_bounds__(T::NT) void mma_kernel(typename XL::Params xp, type
   if constexpr (WS == WS_Y) {
 #pragma unroll
     for (int j = 0; j < T::TY; ++j) wsy[j] += __shfl_xor(wsy[j], 32);
+  }
+
+  if constexpr (T::KG > 1) {
+    // Every k-group must arrive at the same number of workgroup barriers: one in the prologue
+    // and one per stage, for the group with the most stages.
+    const int mine = ke - kb, most = (ke0 - kb0 + T::KG - 1) / T::KG;
+    for (int i = mine > 0 ? 1 + mine : 0; i < 1 + most; ++i) __syncthreads();
+    // Hand the partial sums to the first k-group.  The exchange area lies behind the LDS the
+    // epilogue uses, so a wave that starts its epilogue early cannot overwrite it.
+    constexpr int NW = T::NTG / 64, NB = T::TX * T::TY;
+    char *xch = lds + Epi::template lds_bytes<T>();
+    int *xws = reinterpret_cast<int *>(xch + (T::KG - 1) * (T::BX * T::BY * 4));
+    if (grp > 0) {
+      char *mine_acc = xch + ((grp - 1) * NW + wave) * (NB * 4096);
+      int *mine_ws = xws + ((grp - 1) * NW + wave) * ((T::TX + T::TY) * 64);
+#pragma unroll
+      for (int i = 0; i < T::TX; ++i)
+#pragma unroll
+        for (int j = 0; j < T::TY; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            *reinterpret_cast<typename Op::out4_t *>(mine_acc + (((i * T::TY + j) * 4 + q) * 64 + lane) * 16) =
+                typename Op::out4_t{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+#pragma unroll
+      for (int i = 0; i < T::TX; ++i) mine_ws[i * 64 + lane] = wsx[i];
+#pragma unroll
+      for (int j = 0; j < T::TY; ++j) mine_ws[(T::TX + j) * 64 + lane] = wsy[j];
+    }
+    __syncthreads();
+    if (grp > 0) return;
+#pragma unroll
+    for (int g = 1; g < T::KG; ++g) {
+      const char *its_acc = xch + ((g - 1) * NW + wave) * (NB * 4096);
+      const int *its_ws = xws + ((g - 1) * NW + wave) * ((T::TX + T::TY) * 64);
+#pragma unroll
+      for (int i = 0; i < T::TX; ++i)
+#pragma unroll
+        for (int j = 0; j < T::TY; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const auto v = *reinterpret_cast<const typename Op::out4_t *>(its_acc + (((i * T::TY + j) * 4 + q) * 64 + lane) * 16);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] += v[e];
+          }
+#pragma unroll
+      for (int i = 0; i < T::TX; ++i) wsx[i] += its_ws[i * 64 + lane];
+#pragma unroll
+      for (int j = 0; j < T::TY; ++j) wsy[j] += its_ws[(T::TX + j) * 64 + lane];
+    }
   }
 
   // the last barrier of the K loop came after every LDS read: the tiles are free for the epilogue

@@ -16,8 +16,6 @@ import json
 import os
 import sys
 
-NUM_VARIANTS = 40  # kConvTiles in csrc/conv_plan.hpp
-
 
 def _shapes(spec):
     from . import workloads as WL
@@ -39,6 +37,7 @@ def tune(spec, iters=20, verbose=True, dtype="i8"):
     dev = torch.device("cuda:0")
     L = _lib.load()
     stream = torch.cuda.current_stream().cuda_stream
+    num_variants = L.unit_conv_variant_count()
 
     def time_us(fn):
         for _ in range(3):
@@ -55,7 +54,9 @@ def tune(spec, iters=20, verbose=True, dtype="i8"):
             best = min(best, e0.elapsed_time(e1) * 1e3 / iters)
         return best
 
-    saved = {k: os.environ.get(k) for k in ("UNIT_AMD_CONV_VARIANT", "UNIT_AMD_CONV_SPLITK")}
+    saved = {k: os.environ.get(k) for k in ("UNIT_AMD_CONV_VARIANT", "UNIT_AMD_CONV_SPLITK", "UNIT_AMD_CONV_PANEL",
+                                             "UNIT_AMD_CONV_NOTABLE")}
+    os.environ["UNIT_AMD_CONV_NOTABLE"] = "1"  # "default" below = the heuristic, not an older table
     results = []
     seen = set()
     try:
@@ -90,15 +91,23 @@ def tune(spec, iters=20, verbose=True, dtype="i8"):
 
             os.environ["UNIT_AMD_CONV_VARIANT"] = "0"
             os.environ["UNIT_AMD_CONV_SPLITK"] = "0"
+            os.environ["UNIT_AMD_CONV_PANEL"] = "0"
             _lib.check(call())
             torch.cuda.synchronize()
             ref = out.clone()
             best = (time_us(call), -1, last_variant())
             default_us = best[0]
-            for v in range(NUM_VARIANTS):
-                for splits in ((1, 2, 4, 8, 16, 32) if dtype == "i8" else (1,)):
+            timings = {}  # kernel name -> us, every candidate (kept in the --json dump)
+            combos = [(1, 0), (1, 1), (1, 2), (1, 4)]  # (k-splits, channel tiles per panel)
+            if dtype == "i8":
+                combos += [(n, 0) for n in (2, 4, 8, 16, 32)]
+            for v in range(num_variants):
+                for splits, panel in combos:
+                    if splits > 1 and (splits // 2) * key[0] * s.K > 256 * 256 * 256:
+                        break  # the grid already covers the chip: more k-splits only add atomics
                     os.environ["UNIT_AMD_CONV_VARIANT"] = str(v + 1)
                     os.environ["UNIT_AMD_CONV_SPLITK"] = str(splits)
+                    os.environ["UNIT_AMD_CONV_PANEL"] = str(panel)
                     out.fill_(-7)
                     if call() != 0:  # variant cannot run this shape (LDS budget)
                         break
@@ -106,15 +115,17 @@ def tune(spec, iters=20, verbose=True, dtype="i8"):
                     name = last_variant()
                     if dtype == "i8" and int(name.rsplit("_s", 1)[1]) != splits:
                         break  # clamped to the number of stages: already measured
+                    if panel and f"_r{panel}" not in name:
+                        continue  # fewer channel tiles than the panel: same as panel 0
                     if not torch.equal(out, ref):
                         raise RuntimeError(f"variant {v} ({name}) disagrees with the default on {s.name}")
                     us = time_us(call)
+                    timings[name] = round(us, 2)
                     if us < best[0]:
-                        best = (us, v, name, splits)
-                    if splits * key[0] * s.K > 256 * 256 * 256:
-                        break  # the grid already covers the chip: more k-splits only add atomics
+                        best = (us, v, name, splits, panel)
             results.append(dict(net=net, batch=batch, layer=s.name, key=key, variant=best[1], us=best[0],
-                                default_us=default_us, kernel=best[2], splits=best[3] if len(best) > 3 else 1))
+                                default_us=default_us, kernel=best[2], splits=best[3] if len(best) > 3 else 1,
+                                panel=best[4] if len(best) > 4 else 0, timings=timings))
             if verbose:
                 print(f"{net:9s} b{batch:<3d} {s.name:22s} default {default_us:7.1f} us  best {best[0]:7.1f} us  {best[2]}",
                       flush=True)
@@ -133,7 +144,7 @@ def write_table(results, path):
         if r["variant"] < 0:
             continue  # the heuristic's own choice was the fastest
         npix, k, c, kh, kw, sh = r["key"]
-        lines.append(f"    {{{npix}, {k}, {c}, {kh}, {kw}, {sh}, {r['variant']}, {r['splits']}}},  // {r['net']} b{r['batch']} "
+        lines.append(f"    {{{npix}, {k}, {c}, {kh}, {kw}, {sh}, {r['variant']}, {r['splits']}, {r['panel']}}},  // {r['net']} b{r['batch']} "
                      f"{r['layer']}: {r['us']:.1f} us ({r['kernel']})\n")
     with open(path, "w") as f:
         f.writelines(lines)
