@@ -20,9 +20,12 @@
 
 namespace unit {
 
-template <int TX_, int TY_, int KG_, int D_>
+// PAD: the convolution has zero padding, so taps can fall outside the image and are masked per
+// lane; without it every tap of every valid pixel lies inside and the masking code is left out.
+template <int TX_, int TY_, int KG_, int D_, bool PAD_ = true>
 struct DirectShape {
   static constexpr int TX = TX_, TY = TY_, KG = KG_, D = D_;
+  static constexpr bool PAD = PAD_;
   static constexpr int BX = TX * 32, BY = TY * 32;
   static constexpr int NT = 64 * KG;
   static constexpr int kScratch = ConvEpilogue<OpI8>::kScratch;  // per-wave transpose area
@@ -76,15 +79,16 @@ __global__ __launch_bounds__(S::NT) void conv_direct_i8(const char *__restrict__
   int *wsum = reinterpret_cast<int *>(lds + KG * S::kScratch + S::SUM);
   v2i *tab = reinterpret_cast<v2i *>(lds + S::LDS_FIXED);
 
-  // tap -> (byte offset of the tap inside an image relative to the window origin, window bit);
-  // the odd tap past the end gets bit 0: it is staged like zero padding
+  // tap -> (byte offset of the tap inside an image relative to the window origin, index of its
+  // window position kh * KW + kw); the odd tap past the end points at bit 31 of the window set,
+  // which is never set: it is staged like zero padding
   const int nsteps = (g.ntaps + 1) >> 1;
   for (int e = threadIdx.x; e < 2 * nsteps; e += S::NT) {
-    v2i ent = {0, 0};
+    v2i ent = {0, 31};
     if (e < g.ntaps) {
       const int kw = e % g.KW, rest = e / g.KW, kh = rest % g.KH, ci = rest / g.KH;
       ent[0] = ((ci * g.H + kh * g.dh) * g.W + kw * g.dw) * 16;
-      ent[1] = (int)(1u << (kh * g.KW + kw));
+      ent[1] = kh * g.KW + kw;
     }
     tab[e] = ent;
   }
@@ -140,13 +144,22 @@ __global__ __launch_bounds__(S::NT) void conv_direct_i8(const char *__restrict__
 
   // prefetch ring: D k-steps of fragments in registers
   v4i xf[D][TX], yf[D][TY];
-  int ym[D][TY];  // all ones where the tap lies inside the image, else 0
+  int ym[S::PAD ? D : 1][TY];  // all ones where the tap lies inside the image, else 0
   const u32 last_tap_off = (u32)(g.ntaps - 1) * 256u;
 
-  auto fetch = [&](auto slot, int s) __attribute__((always_inline)) {
+  // Offsets are unsigned 32-bit values added to a uniform base pointer, so a load needs no 64-bit
+  // address arithmetic per lane.
+  // Fetches run through the k-steps in order; `sf` is the next one (it stops at the wave's last
+  // k-step, so surplus fetches re-read that one) and `ecur` its tap table entry, read one fetch
+  // ahead so that the LDS latency is not in the way of the loads.
+  int sf = 0, slast = 0;
+  v2i ecur = {0, 31};
+  auto fetch = [&](auto slot) __attribute__((always_inline)) {
     constexpr int U = decltype(slot)::value;
-    const int t = 2 * s + half;
-    const v2i e = tab[t];
+    const int t = 2 * sf + half;
+    const v2i e = ecur;
+    sf = sf < slast ? sf + 1 : slast;
+    ecur = tab[2 * sf + half];
     // the odd tap past the end re-reads the last tap's weights: its data is staged as zero
     // padding, and a padded position contributes -128 * w to the accumulator and +128 * w through
     // the weight-sum correction, whatever w is
@@ -154,15 +167,20 @@ __global__ __launch_bounds__(S::NT) void conv_direct_i8(const char *__restrict__
     xk = xk < last_tap_off ? xk : last_tap_off;
 #pragma unroll
     for (int i = 0; i < TX; ++i) {
-      const char *p = wgt + xoff[i] + xk;
+      const u32 o = xoff[i] + xk;
 #pragma unroll
-      for (int d = 0; d < 4; ++d) xf[U][i][d] = *reinterpret_cast<const int *>(p + d * 64);
+      for (int d = 0; d < 4; ++d) xf[U][i][d] = *reinterpret_cast<const int *>(wgt + o + d * 64);
     }
 #pragma unroll
     for (int j = 0; j < TY; ++j) {
-      const bool ok = (inside[j] & (u32)e[1]) != 0;
-      yf[U][j] = *reinterpret_cast<const v4i *>(data + (ok ? pixoff[j] + e[0] : 0));
-      ym[U][j] = ok ? -1 : 0;
+      if constexpr (S::PAD) {
+        // all ones if window position e[1] of this lane's pixel is inside the image, else 0
+        const int m = __builtin_amdgcn_sbfe((int)inside[j], (u32)e[1], 1u);
+        yf[U][j] = *reinterpret_cast<const v4i *>(data + ((u32)(pixoff[j] + e[0]) & (u32)m));
+        ym[U][j] = m;
+      } else {
+        yf[U][j] = *reinterpret_cast<const v4i *>(data + (u32)(pixoff[j] + e[0]));
+      }
     }
   };
   auto consume = [&](auto slot) __attribute__((always_inline)) {
@@ -171,7 +189,12 @@ __global__ __launch_bounds__(S::NT) void conv_direct_i8(const char *__restrict__
 #pragma unroll
     for (int j = 0; j < TY; ++j)
 #pragma unroll
-      for (int d = 0; d < 4; ++d) y[j][d] = (yf[U][j][d] & ym[U][j]) ^ (int)0x80808080;
+      for (int d = 0; d < 4; ++d) {
+        if constexpr (S::PAD)
+          y[j][d] = (yf[U][j][d] & ym[U][j]) ^ (int)0x80808080;
+        else
+          y[j][d] = yf[U][j][d] ^ (int)0x80808080;
+      }
 #pragma unroll
     for (int i = 0; i < TX; ++i)
 #pragma unroll
@@ -181,50 +204,57 @@ __global__ __launch_bounds__(S::NT) void conv_direct_i8(const char *__restrict__
 #pragma unroll
       for (int j = 0; j < TY; ++j) acc[i][j] = OpI8::mma(xf[U][i], y[j], acc[i][j]);
   };
-  // D consecutive k-steps starting at s, slots resolved at compile time
-  auto ring = [&](int s, int s1, auto steady) __attribute__((always_inline)) {
-    auto one = [&](auto u) __attribute__((always_inline)) {
-      constexpr int UU = decltype(u)::value;
-      if constexpr (decltype(steady)::value) {
-        consume(u);
-        fetch(u, s + UU + D);
-      } else {
-        if (s + UU < s1) {
-          consume(u);
-          if (s + UU + D < s1) fetch(u, s + UU + D);
-        }
-      }
-    };
-    one(std::integral_constant<int, 0>{});
-    one(std::integral_constant<int, 1>{});
-    if constexpr (D > 2) one(std::integral_constant<int, 2>{});
-    if constexpr (D > 3) one(std::integral_constant<int, 3>{});
-    if constexpr (D > 4) one(std::integral_constant<int, 4>{});
-    if constexpr (D > 5) one(std::integral_constant<int, 5>{});
-    if constexpr (D > 6) one(std::integral_constant<int, 6>{});
-    if constexpr (D > 7) one(std::integral_constant<int, 7>{});
+  // Software pipeline over this wave's k-steps [s0, s1).  Every path issues the same loads in the
+  // same (slot) order and only the consumes are conditional, so the wait the compiler places
+  // before a consume always leaves the D - 1 younger slots in flight.  (With conditional
+  // fetches the wait has to cover the path on which the slot is the youngest load and becomes
+  // "wait for everything".)  The price: fetches past the end re-read the last k-step.
+  // The sched_barriers keep consume(u) -> fetch(u) in program order; left alone, the scheduler
+  // gathers the loads of all D slots at the end of the loop body.
+  auto for_slots = [&](auto f) __attribute__((always_inline)) {
+    f(std::integral_constant<int, 0>{});
+    f(std::integral_constant<int, 1>{});
+    if constexpr (D > 2) f(std::integral_constant<int, 2>{});
+    if constexpr (D > 3) f(std::integral_constant<int, 3>{});
+    if constexpr (D > 4) f(std::integral_constant<int, 4>{});
+    if constexpr (D > 5) f(std::integral_constant<int, 5>{});
+    if constexpr (D > 6) f(std::integral_constant<int, 6>{});
+    if constexpr (D > 7) f(std::integral_constant<int, 7>{});
   };
 
   __syncthreads();  // tap table (and the zeroed sums) visible
 
   const int s0 = nsteps * wave / KG, s1 = nsteps * (wave + 1) / KG;
-  {
-    auto pre = [&](auto u) __attribute__((always_inline)) {
-      constexpr int UU = decltype(u)::value;
-      if (s0 + UU < s1) fetch(u, s0 + UU);
-    };
-    pre(std::integral_constant<int, 0>{});
-    pre(std::integral_constant<int, 1>{});
-    if constexpr (D > 2) pre(std::integral_constant<int, 2>{});
-    if constexpr (D > 3) pre(std::integral_constant<int, 3>{});
-    if constexpr (D > 4) pre(std::integral_constant<int, 4>{});
-    if constexpr (D > 5) pre(std::integral_constant<int, 5>{});
-    if constexpr (D > 6) pre(std::integral_constant<int, 6>{});
-    if constexpr (D > 7) pre(std::integral_constant<int, 7>{});
+  if (s0 < s1) {
+    sf = s0;
+    slast = s1 - 1;
+    ecur = tab[2 * sf + half];
+    for_slots([&](auto u) __attribute__((always_inline)) {
+      fetch(u);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    int s = s0;
+    for (; s + 2 * D <= s1; s += D)
+      for_slots([&](auto u) __attribute__((always_inline)) {
+        consume(u);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(u);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    if (s + D < s1) {  // D < remaining < 2 D: one more round of fetches (the surplus ones repeat the last k-step)
+      for_slots([&](auto u) __attribute__((always_inline)) {
+        consume(u);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(u);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      s += D;
+    }
+    for_slots([&](auto u) __attribute__((always_inline)) {  // 1 .. D k-steps left, all in flight
+      if (s + decltype(u)::value < s1) consume(u);
+      __builtin_amdgcn_sched_barrier(0);
+    });
   }
-  int s = s0;
-  for (; s + 2 * D <= s1; s += D) ring(s, s1, std::true_type{});
-  for (; s < s1; s += D) ring(s, s1, std::false_type{});
 
   // the two 32-lane halves hold the weight sums of the two taps of every k-step
 #pragma unroll

@@ -30,7 +30,7 @@ int run_direct(const unit_conv_desc *d, const ConvGeom &g, const void *data, con
   gm.total = gm.gx * gm.gy;
   char tail[16] = "";
   if (panel) snprintf(tail, sizeof tail, "_r%d", panel);
-  set_variant("i8direct_c16_x%d_y%d_g%d_d%d%s_s1", S::BX, S::BY, S::KG, S::D, tail);
+  set_variant("i8direct_c16_x%d_y%d_g%d_d%d%s%s_s1", S::BX, S::BY, S::KG, S::D, S::PAD ? "" : "n", tail);
   hipLaunchKernelGGL(kern, dim3(gm.total), dim3(S::NT), lds, s, static_cast<const char *>(data),
                      static_cast<const char *>(w), ep, g, gm);
   hipError_t e = hipGetLastError();
@@ -42,13 +42,17 @@ int run_direct(const unit_conv_desc *d, const ConvGeom &g, const void *data, con
 
 int conv_i8_direct(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
                    void *out, hipStream_t s) {
-  if (d->cb != 16 || d->KH * d->KW > 32)
+  if (d->cb != 16 || d->KH * d->KW > 31)
     return fail(UNIT_E_ARG, "unit_conv2d_nchwc_u8s8s32: kernel variant %d not available for this layout or window",
                 plan.variant);
+  // Without zero padding every tap of a valid pixel lies inside the image and the kernel without
+  // tap masks serves; an odd tap count needs the masks too, for the tap that pads the last k-step.
+  const bool masked = d->pt || d->pl || d->pb || d->pr || (g.ntaps & 1);
 #define UNIT_CONV_VARIANT(ID, BX, BY, BKB, WX, WY, PF, FF, KG)
 #define UNIT_CONV_DIRECT(ID, TX, TY, KG, D) \
   case ID:                                  \
-    return run_direct<DirectShape<TX, TY, KG, D>>(d, g, data, w, out, plan, s);
+    return masked ? run_direct<DirectShape<TX, TY, KG, D, true>>(d, g, data, w, out, plan, s) \
+                  : run_direct<DirectShape<TX, TY, KG, D, false>>(d, g, data, w, out, plan, s);
   switch (plan.variant) {
 #include "conv_variants.def"
     default:
