@@ -81,6 +81,10 @@ int conv_geom(const unit_conv_desc *d, int tapb, ConvGeom *g, const char *what) 
   g->ntaps = cc * d->KH * d->KW;
   g->ntab = g->ntaps;
   g->img_bytes = (u32)img;
+  g->by_ohw = FastDiv::make(OH * OW);
+  g->by_ow = FastDiv::make(OW);
+  g->by_kh = FastDiv::make(d->KH);
+  g->by_kw = FastDiv::make(d->KW);
   return UNIT_OK;
 }
 

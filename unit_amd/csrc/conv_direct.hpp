@@ -53,7 +53,8 @@ __device__ __forceinline__ void store_block_i8(const ConvEpilogue<OpI8>::Params 
 #pragma unroll
   for (int it = 0; it < 2; ++it) {
     const int m = m0 + it * 16 + rp;
-    const int n = m / p.ohw, pix = m - n * p.ohw;
+    int n, pix;
+    p.by_ohw.divmod(m, n, pix);
     const size_t obase = ((size_t)n * ko_planes * p.ohw + pix) * 16 + piece * 4;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
@@ -86,7 +87,9 @@ __global__ __launch_bounds__(S::NT) void conv_direct_i8(const char *__restrict__
   for (int e = threadIdx.x; e < 2 * nsteps; e += S::NT) {
     v2i ent = {0, 31};
     if (e < g.ntaps) {
-      const int kw = e % g.KW, rest = e / g.KW, kh = rest % g.KH, ci = rest / g.KH;
+      int kw, rest, kh, ci;
+      g.by_kw.divmod(e, rest, kw);
+      g.by_kh.divmod(rest, ci, kh);
       ent[0] = ((ci * g.H + kh * g.dh) * g.W + kw * g.dw) * 16;
       ent[1] = kh * g.KW + kw;
     }
@@ -119,14 +122,15 @@ __global__ __launch_bounds__(S::NT) void conv_direct_i8(const char *__restrict__
     pixoff[j] = 0;
     inside[j] = 0;
     if (m < g.npix) {
-      const int n = m / (g.OH * g.OW), rem = m - n * (g.OH * g.OW);
-      const int oh = rem / g.OW, ow = rem - oh * g.OW;
+      int n, rem, oh, ow;
+      g.by_ohw.divmod(m, n, rem);
+      g.by_ow.divmod(rem, oh, ow);
       const int ih0 = oh * g.sh - g.pt, iw0 = ow * g.sw - g.pl;
       pixoff[j] = (int)(n * g.img_bytes) + (ih0 * g.W + iw0) * 16;
-      u32 bits = 0;
+      u32 cols = 0, bits = 0;  // columns kw inside the image; then one copy of them per row kh inside
+      for (int kw = 0; kw < g.KW; ++kw) cols |= (u32)((u32)(iw0 + kw * g.dw) < (u32)g.W) << kw;
       for (int kh = 0; kh < g.KH; ++kh)
-        for (int kw = 0; kw < g.KW; ++kw)
-          if ((u32)(ih0 + kh * g.dh) < (u32)g.H && (u32)(iw0 + kw * g.dw) < (u32)g.W) bits |= 1u << (kh * g.KW + kw);
+        if ((u32)(ih0 + kh * g.dh) < (u32)g.H) bits |= cols << (kh * g.KW);
       inside[j] = bits;
     }
   }

@@ -20,7 +20,7 @@ int run_direct(const unit_conv_desc *d, const ConvGeom &g, const void *data, con
     if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "%s: hipFuncSetAttribute: %s", what, hipGetErrorString(e));
     lds_allowed = kMaxLds;
   }
-  ConvEpilogue<OpI8>::Params ep{out, d->K, g.OH * g.OW, g.npix};
+  ConvEpilogue<OpI8>::Params ep{out, d->K, g.OH * g.OW, g.npix, g.by_ohw};
   GridMap gm;
   gm.gx = ceil_div(d->K, S::BX);
   gm.gy = ceil_div(g.npix, S::BY);

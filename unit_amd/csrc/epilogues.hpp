@@ -68,6 +68,7 @@ struct ConvEpilogue {
     int K;     // output channels (multiple of 16)
     int ohw;   // OH * OW
     int npix;  // N * OH * OW
+    FastDiv by_ohw;
   };
   static constexpr int kPitch = 144;               // bytes per pixel row of the scratch
   static constexpr int kScratch = 32 * kPitch;     // per wave
@@ -103,7 +104,8 @@ struct ConvEpilogue {
       for (int it = 0; it < 2; ++it) {
         const int m = yw0 + j * 32 + it * 16 + rp;
         ok[it] = m < p.npix;
-        const int n = m / p.ohw, pix = m - n * p.ohw;
+        int n, pix;
+        p.by_ohw.divmod(m, n, pix);
         obase[it] = ((size_t)n * ko_planes * p.ohw + pix) * 16 + piece * 4;
       }
 #pragma unroll

@@ -237,6 +237,7 @@ struct ConvGeom {
   int ntaps;   // (C / cb) * KH * KW
   int ntab;    // table entries (ntaps rounded up to whole pipeline stages)
   u32 img_bytes;  // bytes per image
+  FastDiv by_ohw, by_ow, by_kh, by_kw;  // dividers by OH * OW, OW, KH, KW
 };
 
 template <int ROWS, int BKB, int NT, int TAPB, bool XOR80, int PF = 1>
@@ -272,7 +273,9 @@ struct ConvPixelLoader {
     for (int e = t; e < g.ntab; e += NT) {
       v2i ent;
       if (e < g.ntaps) {
-        const int kw = e % g.KW, rest = e / g.KW, kh = rest % g.KH, ci = rest / g.KH;
+        int kw, rest, kh, ci;
+        g.by_kw.divmod(e, rest, kw);
+        g.by_kh.divmod(rest, ci, kh);
         ent[0] = ((ci * g.H + kh * g.dh) * g.W + kw * g.dw) * TAPB;
         ent[1] = (kh * g.dh) | ((kw * g.dw) << 16);
       } else {
@@ -287,8 +290,9 @@ struct ConvPixelLoader {
     for (int s = 0; s < PPT; ++s) {
       const int m = row0 + prow + s * NT;
       if (m < g.npix) {
-        const int n = m / (g.OH * g.OW), rem = m - n * (g.OH * g.OW);
-        const int oh = rem / g.OW, ow = rem - oh * g.OW;
+        int n, rem, oh, ow;
+        g.by_ohw.divmod(m, n, rem);
+        g.by_ow.divmod(rem, oh, ow);
         ih0[s] = oh * g.sh - g.pt;
         iw0[s] = ow * g.sw - g.pl;
         pixoff[s] = (int)(n * g.img_bytes) + (ih0[s] * g.W + iw0[s]) * TAPB;

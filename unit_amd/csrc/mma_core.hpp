@@ -52,6 +52,28 @@ struct OpF16 {
   }
 };
 
+// Division of a 31-bit dividend by a runtime constant: q = mulhi(2 n, mul) >> shift with
+// shift = ceil(log2 d) and mul = floor(2^(31 + shift) / d) + 1 (2^31 for a power of two), which
+// is exact for 0 <= n < 2^31.  Three instructions instead of the ~35 of an integer division;
+// pixel and tap indices are decoded this way in kernel prologues and epilogues.
+struct FastDiv {
+  u32 mul, shift;
+  int d;
+  __host__ static FastDiv make(int d) {
+    FastDiv f;
+    f.d = d;
+    f.shift = 0;
+    while ((1u << f.shift) < (u32)d) ++f.shift;
+    f.mul = ((1u << f.shift) == (u32)d) ? 0x80000000u : (u32)((1ull << (31 + f.shift)) / (unsigned long long)d) + 1u;
+    return f;
+  }
+  __device__ __forceinline__ int div(int n) const { return (int)(__umulhi((u32)n << 1, mul) >> shift); }
+  __device__ __forceinline__ void divmod(int n, int &q, int &r) const {
+    q = div(n);
+    r = n - q * d;
+  }
+};
+
 // XOR mask for the 16-byte chunk index of an LDS row.  Chosen so that any 8 (32 banks) or 16
 // (64 banks) consecutive rows reading the same logical chunk land on distinct banks, for rows
 // of 128 bytes (8 chunks) and of 64 bytes (4 chunks).
