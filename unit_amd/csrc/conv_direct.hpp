@@ -61,7 +61,7 @@ __device__ __forceinline__ void store_block_i8(const ConvEpilogue<OpI8>::Params 
       const int c = c0 + h * 16;
       const v4i v = *reinterpret_cast<const v4i *>(scratch + (it * 16 + rp) * kPitch + h * 64 + piece * 16);
       if (c < p.K && m < p.npix)
-        *reinterpret_cast<v4i *>(reinterpret_cast<int *>(p.out) + obase + (size_t)(c >> 4) * p.ohw * 16) = v;
+        __builtin_nontemporal_store(v, reinterpret_cast<v4i *>(reinterpret_cast<int *>(p.out) + obase + (size_t)(c >> 4) * p.ohw * 16));
     }
   }
 }
