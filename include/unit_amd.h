@@ -74,6 +74,20 @@ int unit_conv_out_hw(const unit_conv_desc *d, int32_t *OH, int32_t *OW);
 int unit_conv2d_nchwc_u8s8s32(const unit_conv_desc *d, const void *data, const void *weight,
                               void *out, unit_stream_t stream);
 
+/* The convolution as the reference's quantized models run it,
+ * fused_nn_contrib_conv2d_NCHWc_subtract_add_multiply (apps/cpu/relay/result.log:3-26,35):
+ * signed activations x are shifted to u8 (x + 128), convolved, corrected by 128 * sum(w) per
+ * output channel, biased and scaled:
+ *   out = (conv_u8(x + 128, w) - 128 * sum_{c,kh,kw} w[k] + bias[k]) * scale      (all int32)
+ * which equals (sum x * w + bias[k]) * scale on the signed data; the signed MFMA computes that
+ * directly, with neither the shift nor the correction.
+ *   data   s8  (N, C/cb, H, W, cb)
+ *   weight s8  (K/16, C/cb, KH, KW, cb/4, 16, 4)
+ *   bias   i32 (K) or NULL;  scale: int32 factor (the reference prints 11)
+ *   out    i32 (N, K/16, OH, OW, 16) */
+int unit_conv2d_nchwc_s8s8s32_fused(const unit_conv_desc *d, const void *data, const void *weight,
+                                    const int32_t *bias, int32_t scale, void *out, unit_stream_t stream);
+
 /* topi.x86.dense_dotprod(data, weight, None, 'int32') as called at
  * apps/cpu/kernel/int8-gemm.py:13-16.
  *   a   u8  (M, K) row-major

@@ -209,6 +209,30 @@ def conv2d_nchwc_int8_loops(data, weight, stride=1, padding=0, dilation=1):
     return (out & 0xFFFFFFFF).astype(np.uint32).view(np.int32)
 
 
+def conv2d_nchwc_int8_fused(data_s8, weight, bias, scale, stride=1, padding=0, dilation=1, conv=None):
+    """fused_nn_contrib_conv2d_NCHWc_subtract_add_multiply, op by op as the reference prints it
+    (apps/cpu/relay/result.log:3-26): x + 128 cast to u8 (:4-6), the u8 x s8 convolution (:14),
+    minus 128 * sum of the weights over (in-channel, kh, kw) per out channel (:15-21), plus the bias
+    (:22-23), times the scale (:24), in wrapping int32.  The printed graphs carry no spatial padding;
+    a padded convolution is taken as upstream TVM legalises it: zero-pad the signed data first,
+    then shift, so the correction stays exact at the borders.  `conv` is the u8 convolution to use
+    (default: the vectorised numpy restatement)."""
+    data_s8 = np.asarray(data_s8)
+    weight = np.asarray(weight)
+    assert data_s8.dtype == np.int8 and weight.dtype == np.int8
+    pt, pl, pb, pr = _pad_tuple(padding)
+    xp = np.pad(data_s8, ((0, 0), (0, 0), (pt, pb), (pl, pr), (0, 0)))
+    xu = (xp.astype(np.int32) + 128).astype(np.uint8)
+    conv = conv or conv2d_nchwc_int8
+    acc = conv(xu, weight, stride, 0, dilation).astype(np.int64)             # (N, K/16, OH, OW, 16)
+    wsum = weight.astype(np.int64).sum(axis=(1, 2, 3, 4, 6))                  # (K/16, 16)
+    out = acc - 128 * wsum[None, :, None, None, :]
+    if bias is not None:
+        out = out + np.asarray(bias, dtype=np.int64).reshape(1, -1, 1, 1, 16)
+    out = out * int(scale)
+    return np.ascontiguousarray((out & 0xFFFFFFFF).astype(np.uint32).view(np.int32))
+
+
 # --------------------------------------------------------------------------- a3 dense
 def dense_logical(a, w):
     """relay.nn.dense(x, w) of apps/cpu/relay/int8-gemm.py:14-16: C = A . W^T, A u8 (M,K), W s8 (N,K)."""

@@ -140,6 +140,51 @@ def test_conv2d_every_variant(dev, oracle, monkeypatch, N, C, H, W, K, ks, strid
     assert len({name for _, name in ran}) >= len({v for v, _ in ran}) >= 46
 
 
+FUSED_CASES = [
+    # N, C, H, W, K, kernel, stride, pad, with bias
+    (1, 1024, 16, 16, 2048, 1, 1, 0, True),     # apps/cpu/relay/result.log:3-26
+    (1, 3, 224, 224, 64, 7, 2, 0, True),        # result.log:6803-6828 (channels padded to 4: NCHW4c)
+    (2, 64, 14, 14, 96, 3, 1, 1, True),         # zero padding in the signed domain
+    (3, 48, 9, 11, 80, 3, 2, (1, 0, 2, 1), False),
+    (32, 256, 14, 14, 256, 3, 1, 1, True),      # ResNet-50 batch 32 layer
+    (1, 16, 20, 20, 32, 7, 1, 3, True),         # 49-position window on NCHW16c: staged kernel
+    (2, 32, 5, 5, 16, 1, 1, 0, False),          # one k-step
+]
+
+
+@pytest.mark.parametrize("N,C,H,W,K,ks,stride,pad,with_bias", FUSED_CASES)
+def test_conv2d_fused_bit_exact(dev, oracle, N, C, H, W, K, ks, stride, pad, with_bias):
+    """(conv(x_s8 + 128, w) - 128 sum(w) + bias) * scale of the reference's quantized graphs."""
+    cb = 16 if C % 16 == 0 else 4
+    x = oracle.pack_nchwc(rng.uniform_s8((N, C, H, W), 13 * C + H), cb)
+    wt = rng.uniform_s8((K // 16, x.shape[1], ks, ks, cb // 4, 16, 4), 7 * K + ks)
+    bias = (rng.uniform_s8((K,), 5).astype(np.int32) * 4099) if with_bias else None
+    ref = oracle.conv2d_nchwc_int8_fused(x, wt, bias, 11, stride, pad, 1, conv=oracle.c_conv2d_nchwc)
+    out = U.conv2d_NCHWc_int8_fused(_t(x, dev), _t(wt, dev), _t(bias, dev) if with_bias else None, 11, stride, pad, 1,
+                                    "int32", f"NCHW{cb}c", "NCHW16c")
+    torch.cuda.synchronize()
+    assert tuple(out.shape) == ref.shape
+    assert np.array_equal(out.cpu().numpy(), ref), U.last_variant()
+
+
+def test_conv2d_fused_every_direct_variant(dev, oracle, monkeypatch):
+    from unit_amd import _lib
+    N, C, H, W, K, ks = 2, 80, 9, 11, 96, 3
+    x = rng.uniform_s8((N, C // 16, H, W, 16), 3)
+    wt = rng.uniform_s8((K // 16, C // 16, ks, ks, 4, 16, 4), 4)
+    bias = rng.uniform_s8((K,), 5).astype(np.int32) * 77
+    ref = oracle.conv2d_nchwc_int8_fused(x, wt, bias, -3, 1, 1, 1, conv=oracle.c_conv2d_nchwc)
+    tx, tw, tb = _t(x, dev), _t(wt, dev), _t(bias, dev)
+    names = set()
+    for v in range(1, _lib.load().unit_conv_variant_count() + 1):
+        monkeypatch.setenv("UNIT_AMD_CONV_VARIANT", str(v))
+        out = U.conv2d_NCHWc_int8_fused(tx, tw, tb, -3, 1, 1)
+        torch.cuda.synchronize()
+        names.add(U.last_variant())
+        assert np.array_equal(out.cpu().numpy(), ref), (v, U.last_variant())
+    assert len(names) >= 15 and all(n.startswith("s8direct") for n in names)
+
+
 def test_conv2d_zero_padding_value(dev, oracle):
     """Padded pixels are u8 zeros: with all-255 data and all-ones weights every output equals
     255 * (number of in-image taps) * C, which differs between border and interior."""

@@ -232,6 +232,45 @@ def test_unsigned_to_signed_shift_identity(oracle):
     assert np.array_equal(signed + corr, ref.astype(np.float64))
 
 
+@pytest.mark.parametrize("cb,ks,stride,pad", [(16, 1, 1, 0), (16, 3, 1, 1), (4, 7, 2, 3), (16, 3, 2, (0, 1, 1, 0))])
+def test_fused_form_is_the_signed_convolution(oracle, cb, ks, stride, pad):
+    """The reference's fused graph (x + 128 -> u8 conv -> - 128 sum(w) -> + bias -> * scale,
+    apps/cpu/relay/result.log:3-26) equals (signed conv + bias) * scale, computed here by an
+    independent routine (torch float64 conv2d on the un-blocked tensors, exact at these sizes)."""
+    n, c, hw, k = 2, 2 * cb, 9, 32
+    x = oracle.fill_s8((n, c, hw, hw), 41)
+    w = oracle.fill_s8((k, c, ks, ks), 42)
+    b = (oracle.fill_s8((k,), 43).astype(np.int32) * 1000)
+    pt, pl, pb, pr = (pad,) * 4 if isinstance(pad, int) else pad
+    xt = torch.nn.functional.pad(torch.from_numpy(x).double(), (pl, pr, pt, pb))
+    signed = torch.nn.functional.conv2d(xt, torch.from_numpy(w).double(), stride=stride).numpy()
+    want = ((signed + b.reshape(1, k, 1, 1)) * 11).astype(np.int64)
+    for conv in (None, oracle.c_conv2d_nchwc):
+        got = oracle.conv2d_nchwc_int8_fused(oracle.pack_nchwc(x, cb), oracle.prepack_conv_weight(w, cb), b, 11,
+                                             stride, pad, 1, conv=conv)
+        assert np.array_equal(oracle.unpack_nchwc(got, k).astype(np.int64), want)
+
+
+def test_fused_form_printed_shapes(oracle):
+    """The two graphs the reference prints: 1x1 1024 -> 2048 on 16x16 (result.log:3-26) and the 7x7
+    stride-2 stem 3 -> 64 on 224x224 with the input channels padded to 4 (result.log:6803-6828),
+    scale 11; reduced in size here (same structure), checked against int64 loops on the signed data."""
+    for (c, k, hw, ks, stride, cb) in ((32, 32, 5, 1, 1, 16), (3, 16, 19, 7, 2, 4)):
+        x = oracle.fill_s8((1, c, hw, hw), 51)
+        w = oracle.fill_s8((k, c, ks, ks), 52)
+        b = oracle.fill_s8((k,), 53).astype(np.int32)
+        got = oracle.unpack_nchwc(oracle.conv2d_nchwc_int8_fused(oracle.pack_nchwc(x, cb), oracle.prepack_conv_weight(w, cb),
+                                                                  b, 11, stride, 0, 1), k)
+        oh = (hw - ks) // stride + 1
+        want = np.zeros((1, k, oh, oh), dtype=np.int64)
+        for o in range(k):
+            for y in range(oh):
+                for z in range(oh):
+                    win = x[0, :, y * stride:y * stride + ks, z * stride:z * stride + ks].astype(np.int64)
+                    want[0, o, y, z] = ((win * w[o].astype(np.int64)).sum() + b[o]) * 11
+        assert np.array_equal(got.astype(np.int64), want)
+
+
 # ------------------------------------------------------------------ a8 / a9
 def test_fp16_golden_and_integer_exact(oracle):
     g = np.load(os.path.join(GOLD, "fp16_gemm_24x36x40.npz"))

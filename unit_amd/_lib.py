@@ -17,6 +17,7 @@ SYMBOLS = (
     "unit_conv_variant_count",
     "unit_conv_out_hw",
     "unit_conv2d_nchwc_u8s8s32",
+    "unit_conv2d_nchwc_s8s8s32_fused",
     "unit_dense_dotprod_u8s8s32",
     "unit_dense_u8s8s32",
     "unit_gemm_f16",
@@ -62,6 +63,7 @@ def load():
     L.unit_last_variant.restype = ctypes.c_char_p
     L.unit_conv_out_hw.argtypes = [dp, ctypes.POINTER(i32), ctypes.POINTER(i32)]
     L.unit_conv2d_nchwc_u8s8s32.argtypes = [dp, vp, vp, vp, vp]
+    L.unit_conv2d_nchwc_s8s8s32_fused.argtypes = [dp, vp, vp, vp, i32, vp, vp]
     L.unit_dense_dotprod_u8s8s32.argtypes = [vp, vp, vp, i32, i32, i32, vp]
     L.unit_dense_u8s8s32.argtypes = [vp, vp, vp, i32, i32, i32, vp]
     L.unit_gemm_f16.argtypes = [vp, vp, vp, i32, i32, i32, i32, vp]

@@ -1,19 +1,28 @@
-// int8 NCHW16c convolution with both MFMA operands read straight from global memory into
-// registers: no operand staging in LDS, no barrier in the reduction loop.
+// NCHW16c convolution with both MFMA operands read straight from global memory into registers:
+// no operand staging in LDS, no barrier in the reduction loop.
 //
 // Why: staging costs an LDS write and (wave tile permitting) several LDS reads per operand byte,
 // all through one 64-byte-per-clock pipe, and that pipe -- not the matrix cores -- bounds the
 // staged kernel whenever the output tile is small.  The layouts the reference uses happen to be
-// MFMA fragments already:
-//   * data (N, C/16, H, W, 16) u8: the 16 channels of one pixel and tap are 16 contiguous bytes
-//     = one lane's share of a k-step; consecutive lanes hold consecutive pixels (coalesced);
-//   * weights (K/16, C/16, KH, KW, 4, 16, 4) s8: for one tap, channel kb of a 16-channel block owns
-//     dwords at kb*4 + e*64, e = 0..3: four dword loads per lane, 64-byte runs per 16 lanes.
-// One k-step (32 reduction bytes per row) = two taps: lanes 0-31 hold tap 2s, lanes 32-63 tap 2s+1.
+// MFMA fragments already (a lane holds 16 reduction bytes of one row per k-step):
+//   * int8 data (N, C/16, H, W, 16) u8 / s8: the 16 channels of one pixel and tap are 16
+//     contiguous bytes; consecutive lanes hold consecutive pixels (coalesced).  One k-step (32
+//     bytes per row) = two taps: lanes 0-31 hold tap 2s, lanes 32-63 tap 2s+1;
+//   * int8 weights (K/16, C/16, KH, KW, 4, 16, 4) s8: for one tap, channel kb of a 16-channel
+//     block owns the dwords at kb*4 + e*64, e = 0..3: four dword loads per lane;
+//   * fp16 data (N, C/16, H, W, 16): a pixel and tap are 32 bytes = one k-step; lanes 0-31 take
+//     channels 0-7, lanes 32-63 channels 8-15;
+//   * fp16 weights (K/16, C/16, KH, KW, 16 in, 16 out): out-channel o of a tap owns the halves at
+//     o*2 + i*32: eight 16-bit loads per lane, packed in pairs by the load instruction.
 //
 // A workgroup is KG waves that all compute the same (32 TX channels) x (32 TY pixels) tile, each
 // over its own share of the k-steps with a D-deep register prefetch ring; the partial tiles are
-// summed in LDS (integer adds: exact in any order) and the waves share the write-back.
+// summed in LDS and the waves share the write-back.
+//
+// The u8 operand is shifted to s8 (x ^ 0x80) for the signed MFMA and the kernel adds back
+// 128 * sum(w), accumulated on the side with v_dot4 (SHIFT).  Signed data needs neither; that is
+// the reference's fused form  (conv(x_s8 + 128, w) - 128 * sum(w) + bias) * scale
+// (apps/cpu/relay/result.log:3-26), which the epilogue's bias and scale complete.
 #pragma once
 #include "epilogues.hpp"
 #include "loaders.hpp"
@@ -28,26 +37,38 @@ struct DirectShape {
   static constexpr bool PAD = PAD_;
   static constexpr int BX = TX * 32, BY = TY * 32;
   static constexpr int NT = 64 * KG;
-  static constexpr int kScratch = ConvEpilogue<OpI8>::kScratch;  // per-wave transpose area
-  static constexpr int SUM = TX * TY * 4096;                     // summed tile (KG > 1)
-  static constexpr int WSUM = TX * 32 * 4;                       // summed 128 * weight sums
-  static constexpr int LDS_FIXED = KG * kScratch + SUM + WSUM;   // the tap table follows
+  static constexpr int kScratch = 32 * 144;       // per-wave transpose area (32 pixels x 144-byte pitch)
+  static constexpr int TILE = TX * TY * 4096;     // one 4-byte accumulator tile
+  static constexpr int WSUM = TX * 32 * 4;        // summed 128 * weight sums
+  // integer partial tiles are added into one LDS tile with atomics (exact in any order); float
+  // ones are kept apart, one per wave, and summed in wave order so that results do not vary
+  template <class Op>
+  static constexpr int lds_fixed() {
+    return KG * kScratch + (KG > 1 ? (Op::kInt ? TILE : KG * TILE) : 0) + WSUM;  // the tap table follows
+  }
   static_assert(NT <= 1024 && D >= 2 && D <= 8, "direct conv shape");
 };
 
-// Write one 32-channel x 32-pixel accumulator block (plus the per-channel correction in
-// wsb[32], LDS) to the (N, K/16, OH, OW, 16) output: transposed through the wave's LDS scratch so
-// that 64 lanes store 16 pixels x 64 bytes = 1 KiB of consecutive output per instruction.
-__device__ __forceinline__ void store_block_i8(const ConvEpilogue<OpI8>::Params &p, const v16i &acc, const int *wsb,
-                                               int c0, int m0, int lane, char *scratch) {
-  constexpr int kPitch = ConvEpilogue<OpI8>::kPitch;
+// Write one 32-channel x 32-pixel accumulator block to the (N, K/16, OH, OW, 16) output:
+// transposed through the wave's LDS scratch so that 64 lanes store 16 pixels x 64 bytes = 1 KiB of
+// consecutive output per instruction.  `wsb` (LDS, 32 values, or null) holds what is added per
+// channel before the scale: the 128 * sum(w) correction and / or the bias.
+template <class Op>
+__device__ __forceinline__ void store_block(const typename ConvEpilogue<Op>::Params &p, const typename Op::acc_t &acc,
+                                            const int *wsb, int scale, int c0, int m0, int lane, char *scratch) {
+  using out4_t = typename Op::out4_t;
+  using out_t = typename Op::out_t;
+  constexpr int kPitch = 144;
   const int l32 = lane & 31, half = lane >> 5;
   const int rp = lane >> 2, piece = lane & 3;
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
-    v4i v = {acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]};
-    v += *reinterpret_cast<const v4i *>(wsb + 8 * q + 4 * half);
-    *reinterpret_cast<v4i *>(scratch + l32 * kPitch + (8 * q + 4 * half) * 4) = v;
+    out4_t v = {acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]};
+    if constexpr (Op::kInt) {
+      if (wsb) v += *reinterpret_cast<const v4i *>(wsb + 8 * q + 4 * half);
+      v *= scale;
+    }
+    *reinterpret_cast<out4_t *>(scratch + l32 * kPitch + (8 * q + 4 * half) * 4) = v;
   }
   const int ko_planes = p.K >> 4;
 #pragma unroll
@@ -59,58 +80,65 @@ __device__ __forceinline__ void store_block_i8(const ConvEpilogue<OpI8>::Params 
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int c = c0 + h * 16;
-      const v4i v = *reinterpret_cast<const v4i *>(scratch + (it * 16 + rp) * kPitch + h * 64 + piece * 16);
+      const out4_t v = *reinterpret_cast<const out4_t *>(scratch + (it * 16 + rp) * kPitch + h * 64 + piece * 16);
       if (c < p.K && m < p.npix)
-        __builtin_nontemporal_store(v, reinterpret_cast<v4i *>(reinterpret_cast<int *>(p.out) + obase + (size_t)(c >> 4) * p.ohw * 16));
+        __builtin_nontemporal_store(
+            v, reinterpret_cast<out4_t *>(reinterpret_cast<out_t *>(p.out) + obase + (size_t)(c >> 4) * p.ohw * 16));
     }
   }
 }
 
-template <class S>
-__global__ __launch_bounds__(S::NT) void conv_direct_i8(const char *__restrict__ data, const char *__restrict__ wgt,
-                                                        ConvEpilogue<OpI8>::Params ep, ConvGeom g, GridMap gm) {
+template <class Op, class S, bool SHIFT>
+__global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ data, const char *__restrict__ wgt,
+                                                     typename ConvEpilogue<Op>::Params ep, ConvGeom g, GridMap gm) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   constexpr int TX = S::TX, TY = S::TY, KG = S::KG, D = S::D;
+  constexpr bool kInt = Op::kInt;
+  constexpr int TAPB = kInt ? 16 : 32;      // bytes of one pixel and tap
+  constexpr int WTAP = kInt ? 256 : 512;    // bytes of one tap of a 16-channel weight block
+  static_assert(kInt || (!SHIFT && !S::PAD), "the fp16 operator has neither a shift nor padding");
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int l32 = lane & 31, half = lane >> 5;
 
   char *scratch = lds + wave * S::kScratch;
-  int *sum = reinterpret_cast<int *>(lds + KG * S::kScratch);
-  int *wsum = reinterpret_cast<int *>(lds + KG * S::kScratch + S::SUM);
-  v2i *tab = reinterpret_cast<v2i *>(lds + S::LDS_FIXED);
+  char *tiles = lds + KG * S::kScratch;
+  int *wsum = reinterpret_cast<int *>(lds + S::template lds_fixed<Op>() - S::WSUM);
+  v2i *tab = reinterpret_cast<v2i *>(lds + S::template lds_fixed<Op>());
 
   // tap -> (byte offset of the tap inside an image relative to the window origin, index of its
-  // window position kh * KW + kw); the odd tap past the end points at bit 31 of the window set,
-  // which is never set: it is staged like zero padding
-  const int nsteps = (g.ntaps + 1) >> 1;
-  for (int e = threadIdx.x; e < 2 * nsteps; e += S::NT) {
+  // window position kh * KW + kw).  int8 pairs taps into k-steps: the odd tap past the end points
+  // at bit 31 of the window set, which is never set, so it is staged like zero padding.
+  const int nsteps = kInt ? (g.ntaps + 1) >> 1 : g.ntaps;
+  const int ntab = kInt ? 2 * nsteps : nsteps;
+  for (int e = threadIdx.x; e < ntab; e += S::NT) {
     v2i ent = {0, 31};
     if (e < g.ntaps) {
       int kw, rest, kh, ci;
       g.by_kw.divmod(e, rest, kw);
       g.by_kh.divmod(rest, ci, kh);
-      ent[0] = ((ci * g.H + kh * g.dh) * g.W + kw * g.dw) * 16;
+      ent[0] = ((ci * g.H + kh * g.dh) * g.W + kw * g.dw) * TAPB;
       ent[1] = kh * g.KW + kw;
     }
     tab[e] = ent;
   }
-  if constexpr (KG > 1) {
-    for (int e = threadIdx.x; e < (S::SUM + S::WSUM) / 4; e += S::NT) sum[e] = 0;
+  if constexpr (kInt && KG > 1) {
+    int *z = reinterpret_cast<int *>(tiles);
+    for (int e = threadIdx.x; e < (S::TILE + S::WSUM) / 4; e += S::NT) z[e] = 0;
   }
 
   int bx, by, split;
   gm.locate(blockIdx.x, bx, by, split);
   const int x0 = bx * S::BX, y0 = by * S::BY;
 
-  // weights: byte offset of this lane's channel at tap 0, per 32-channel block (rows past K
-  // re-read the last channel; their results are never stored)
+  // weights: byte offset of this lane's share of its channel's tap 0, per 32-channel block (rows
+  // past K re-read the last channel; their results are never stored)
   u32 xoff[TX];
 #pragma unroll
   for (int i = 0; i < TX; ++i) {
     int n = x0 + i * 32 + l32;
     n = n < ep.K ? n : ep.K - 1;
-    xoff[i] = (u32)(n >> 4) * (u32)(g.ntaps * 256) + (u32)(n & 15) * 4u;
+    xoff[i] = (u32)(n >> 4) * (u32)(g.ntaps * WTAP) + (kInt ? (u32)(n & 15) * 4u : (u32)(n & 15) * 2u + (u32)half * 256u);
   }
   // data: byte offset of the window origin of this lane's pixel per 32-pixel block, and the set of
   // window positions (kh, kw) that fall inside the image (none for lanes past the last pixel)
@@ -119,23 +147,25 @@ __global__ __launch_bounds__(S::NT) void conv_direct_i8(const char *__restrict__
 #pragma unroll
   for (int j = 0; j < TY; ++j) {
     const int m = y0 + j * 32 + l32;
-    pixoff[j] = 0;
+    pixoff[j] = kInt ? 0 : half * 16;
     inside[j] = 0;
     if (m < g.npix) {
       int n, rem, oh, ow;
       g.by_ohw.divmod(m, n, rem);
       g.by_ow.divmod(rem, oh, ow);
       const int ih0 = oh * g.sh - g.pt, iw0 = ow * g.sw - g.pl;
-      pixoff[j] = (int)(n * g.img_bytes) + (ih0 * g.W + iw0) * 16;
-      u32 cols = 0, bits = 0;  // columns kw inside the image; then one copy of them per row kh inside
-      for (int kw = 0; kw < g.KW; ++kw) cols |= (u32)((u32)(iw0 + kw * g.dw) < (u32)g.W) << kw;
-      for (int kh = 0; kh < g.KH; ++kh)
-        if ((u32)(ih0 + kh * g.dh) < (u32)g.H) bits |= cols << (kh * g.KW);
-      inside[j] = bits;
+      pixoff[j] += (int)(n * g.img_bytes) + (ih0 * g.W + iw0) * TAPB;
+      if constexpr (S::PAD) {
+        u32 cols = 0, bits = 0;  // columns kw inside the image; then one copy of them per row kh inside
+        for (int kw = 0; kw < g.KW; ++kw) cols |= (u32)((u32)(iw0 + kw * g.dw) < (u32)g.W) << kw;
+        for (int kh = 0; kh < g.KH; ++kh)
+          if ((u32)(ih0 + kh * g.dh) < (u32)g.H) bits |= cols << (kh * g.KW);
+        inside[j] = bits;
+      }
     }
   }
 
-  typename OpI8::acc_t acc[TX][TY];
+  typename Op::acc_t acc[TX][TY];
 #pragma unroll
   for (int i = 0; i < TX; ++i)
 #pragma unroll
@@ -149,31 +179,38 @@ __global__ __launch_bounds__(S::NT) void conv_direct_i8(const char *__restrict__
   // prefetch ring: D k-steps of fragments in registers
   v4i xf[D][TX], yf[D][TY];
   int ym[S::PAD ? D : 1][TY];  // all ones where the tap lies inside the image, else 0
-  const u32 last_tap_off = (u32)(g.ntaps - 1) * 256u;
+  const u32 last_tap_off = (u32)(g.ntaps - 1) * (u32)WTAP;
 
-  // Offsets are unsigned 32-bit values added to a uniform base pointer, so a load needs no 64-bit
-  // address arithmetic per lane.
   // Fetches run through the k-steps in order; `sf` is the next one (it stops at the wave's last
   // k-step, so surplus fetches re-read that one) and `ecur` its tap table entry, read one fetch
   // ahead so that the LDS latency is not in the way of the loads.
+  // Offsets are unsigned 32-bit values added to a uniform base pointer, so a load needs no 64-bit
+  // address arithmetic per lane.
   int sf = 0, slast = 0;
   v2i ecur = {0, 31};
   auto fetch = [&](auto slot) __attribute__((always_inline)) {
     constexpr int U = decltype(slot)::value;
-    const int t = 2 * sf + half;
+    const int t = kInt ? 2 * sf + half : sf;
     const v2i e = ecur;
     sf = sf < slast ? sf + 1 : slast;
-    ecur = tab[2 * sf + half];
-    // the odd tap past the end re-reads the last tap's weights: its data is staged as zero
-    // padding, and a padded position contributes -128 * w to the accumulator and +128 * w through
-    // the weight-sum correction, whatever w is
-    u32 xk = (u32)t * 256u;
+    ecur = tab[kInt ? 2 * sf + half : sf];
+    // int8: the odd tap past the end re-reads the last tap's weights.  Its data is staged as
+    // zero padding, and a padded position contributes -128 * w to the accumulator and +128 * w
+    // through the weight-sum correction (SHIFT) or 0 * w (signed data), whatever w is.
+    u32 xk = (u32)t * (u32)WTAP;
     xk = xk < last_tap_off ? xk : last_tap_off;
 #pragma unroll
     for (int i = 0; i < TX; ++i) {
       const u32 o = xoff[i] + xk;
+      if constexpr (kInt) {
 #pragma unroll
-      for (int d = 0; d < 4; ++d) xf[U][i][d] = *reinterpret_cast<const int *>(wgt + o + d * 64);
+        for (int d = 0; d < 4; ++d) xf[U][i][d] = *reinterpret_cast<const int *>(wgt + o + d * 64);
+      } else {
+        v8h h;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) h[k] = *reinterpret_cast<const _Float16 *>(wgt + o + k * 32);
+        xf[U][i] = __builtin_bit_cast(v4i, h);
+      }
     }
 #pragma unroll
     for (int j = 0; j < TY; ++j) {
@@ -194,19 +231,21 @@ __global__ __launch_bounds__(S::NT) void conv_direct_i8(const char *__restrict__
     for (int j = 0; j < TY; ++j)
 #pragma unroll
       for (int d = 0; d < 4; ++d) {
-        if constexpr (S::PAD)
-          y[j][d] = (yf[U][j][d] & ym[U][j]) ^ (int)0x80808080;
-        else
-          y[j][d] = yf[U][j][d] ^ (int)0x80808080;
+        int v = yf[U][j][d];
+        if constexpr (S::PAD) v &= ym[U][j];
+        if constexpr (SHIFT) v ^= (int)0x80808080;
+        y[j][d] = v;
       }
+    if constexpr (SHIFT) {
+#pragma unroll
+      for (int i = 0; i < TX; ++i)
+#pragma unroll
+        for (int d = 0; d < 4; ++d) wsx[i] = __builtin_amdgcn_sdot4(xf[U][i][d], 0x01010101, wsx[i], false);
+    }
 #pragma unroll
     for (int i = 0; i < TX; ++i)
 #pragma unroll
-      for (int d = 0; d < 4; ++d) wsx[i] = __builtin_amdgcn_sdot4(xf[U][i][d], 0x01010101, wsx[i], false);
-#pragma unroll
-    for (int i = 0; i < TX; ++i)
-#pragma unroll
-      for (int j = 0; j < TY; ++j) acc[i][j] = OpI8::mma(xf[U][i], y[j], acc[i][j]);
+      for (int j = 0; j < TY; ++j) acc[i][j] = Op::mma(xf[U][i], y[j], acc[i][j]);
   };
   // Software pipeline over this wave's k-steps [s0, s1).  Every path issues the same loads in the
   // same (slot) order and only the consumes are conditional, so the wait the compiler places
@@ -232,7 +271,7 @@ __global__ __launch_bounds__(S::NT) void conv_direct_i8(const char *__restrict__
   if (s0 < s1) {
     sf = s0;
     slast = s1 - 1;
-    ecur = tab[2 * sf + half];
+    ecur = tab[kInt ? 2 * sf + half : sf];
     for_slots([&](auto u) __attribute__((always_inline)) {
       fetch(u);
       __builtin_amdgcn_sched_barrier(0);
@@ -261,11 +300,25 @@ __global__ __launch_bounds__(S::NT) void conv_direct_i8(const char *__restrict__
   }
 
   // the two 32-lane halves hold the weight sums of the two taps of every k-step
+  if constexpr (SHIFT) {
 #pragma unroll
-  for (int i = 0; i < TX; ++i) wsx[i] = (wsx[i] + __shfl_xor(wsx[i], 32)) << 7;
+    for (int i = 0; i < TX; ++i) wsx[i] = (wsx[i] + __shfl_xor(wsx[i], 32)) << 7;
+  }
+  // what is added per channel before the scale: the shift correction and / or the bias; one wave
+  // adds the bias.  `addend` is uniform over the workgroup.
+  const bool addend = kInt && (SHIFT || ep.bias != nullptr);
+  if constexpr (kInt) {
+    if (ep.bias != nullptr && wave == 0) {
+#pragma unroll
+      for (int i = 0; i < TX; ++i) {
+        const int c = x0 + i * 32 + l32;
+        wsx[i] += c < ep.K ? ep.bias[c] : 0;
+      }
+    }
+  }
 
   if constexpr (KG == 1) {
-    if (half == 0) {
+    if (addend && half == 0) {
 #pragma unroll
       for (int i = 0; i < TX; ++i) wsum[i * 32 + l32] = wsx[i];
     }
@@ -273,9 +326,11 @@ __global__ __launch_bounds__(S::NT) void conv_direct_i8(const char *__restrict__
     for (int i = 0; i < TX; ++i)
 #pragma unroll
       for (int j = 0; j < TY; ++j)
-        store_block_i8(ep, acc[i][j], wsum + i * 32, x0 + i * 32, y0 + j * 32, lane, scratch);
-  } else {
+        store_block<Op>(ep, acc[i][j], addend ? wsum + i * 32 : nullptr, ep.scale, x0 + i * 32, y0 + j * 32, lane,
+                        scratch);
+  } else if constexpr (kInt) {
     // sum the partial tiles of the KG waves in LDS, then share the blocks among the waves
+    int *sum = reinterpret_cast<int *>(tiles);
 #pragma unroll
     for (int i = 0; i < TX; ++i)
 #pragma unroll
@@ -284,7 +339,7 @@ __global__ __launch_bounds__(S::NT) void conv_direct_i8(const char *__restrict__
         for (int r = 0; r < 16; ++r)
           __hip_atomic_fetch_add(sum + ((i * TY + j) * 16 + r) * 64 + lane, acc[i][j][r], __ATOMIC_RELAXED,
                                  __HIP_MEMORY_SCOPE_WORKGROUP);
-    if (half == 0) {
+    if (addend && half == 0) {
 #pragma unroll
       for (int i = 0; i < TX; ++i)
         __hip_atomic_fetch_add(wsum + i * 32 + l32, wsx[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -295,7 +350,35 @@ __global__ __launch_bounds__(S::NT) void conv_direct_i8(const char *__restrict__
       v16i total;
 #pragma unroll
       for (int r = 0; r < 16; ++r) total[r] = sum[(b * 16 + r) * 64 + lane];
-      store_block_i8(ep, total, wsum + i * 32, x0 + i * 32, y0 + j * 32, lane, scratch);
+      store_block<Op>(ep, total, addend ? wsum + i * 32 : nullptr, ep.scale, x0 + i * 32, y0 + j * 32, lane, scratch);
+    }
+  } else {
+    // float: every wave parks its partial tile; the owner of a block adds them in wave order
+    float *mine = reinterpret_cast<float *>(tiles + wave * S::TILE);
+#pragma unroll
+    for (int i = 0; i < TX; ++i)
+#pragma unroll
+      for (int j = 0; j < TY; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          *reinterpret_cast<v4f *>(mine + (((i * TY + j) * 4 + q) * 64 + lane) * 4) =
+              v4f{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+    __syncthreads();
+    for (int b = wave; b < TX * TY; b += KG) {
+      const int i = b / TY, j = b - i * TY;
+      typename Op::acc_t total;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) total[r] = 0;
+      for (int w = 0; w < KG; ++w) {
+        const float *its = reinterpret_cast<const float *>(tiles + w * S::TILE);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const v4f v = *reinterpret_cast<const v4f *>(its + ((b * 4 + q) * 64 + lane) * 4);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) total[4 * q + e] += v[e];
+        }
+      }
+      store_block<Op>(ep, total, nullptr, 1, x0 + i * 32, y0 + j * 32, lane, scratch);
     }
   }
 }

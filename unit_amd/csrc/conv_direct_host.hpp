@@ -1,0 +1,40 @@
+// Host side of the direct (no operand staging) convolution variants: launch and variant dispatch.
+#pragma once
+#include "conv_direct.hpp"
+#include "conv_plan.hpp"
+
+namespace unit {
+
+template <class Op, class S, bool SHIFT>
+int run_direct(const char *what, const char *tag, const unit_conv_desc *d, const ConvGeom &g, const void *data,
+               const void *w, const int *bias, int scale, void *out, const ConvPlan &plan, hipStream_t s) {
+  const int ntab = Op::kInt ? 2 * ((g.ntaps + 1) / 2) : g.ntaps;
+  const int lds = S::template lds_fixed<Op>() + ntab * 8;
+  if (lds > kMaxLds) return fail(UNIT_E_ARG, "%s: needs %d bytes of LDS (limit %d)", what, lds, kMaxLds);
+  auto kern = conv_direct<Op, S, SHIFT>;
+  static thread_local int lds_allowed = 0;  // the opt-in for > 64 KiB of dynamic LDS is sticky per kernel
+  if (lds > lds_allowed) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
+    if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "%s: hipFuncSetAttribute: %s", what, hipGetErrorString(e));
+    lds_allowed = kMaxLds;
+  }
+  typename ConvEpilogue<Op>::Params ep{out, d->K, g.OH * g.OW, g.npix, g.by_ohw, bias, scale};
+  GridMap gm;
+  gm.gx = ceil_div(d->K, S::BX);
+  gm.gy = ceil_div(g.npix, S::BY);
+  const int panel = plan.panel > 0 && plan.panel < gm.gx ? plan.panel : 0;
+  gm.ph = panel ? panel : gm.gx;
+  gm.splits = 1;
+  gm.total = gm.gx * gm.gy;
+  char tail[16] = "";
+  if (panel) snprintf(tail, sizeof tail, "_r%d", panel);
+  set_variant("%s_x%d_y%d_g%d_d%d%s%s_s1", tag, S::BX, S::BY, S::KG, S::D, S::PAD ? "" : "n", tail);
+  hipLaunchKernelGGL(kern, dim3(gm.total), dim3(S::NT), lds, s, static_cast<const char *>(data),
+                     static_cast<const char *>(w), ep, g, gm);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "%s: launch: %s", what, hipGetErrorString(e));
+  return UNIT_OK;
+}
+
+}  // namespace unit

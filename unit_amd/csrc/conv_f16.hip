@@ -7,6 +7,8 @@
 namespace unit {
 
 int conv_geom(const unit_conv_desc *d, int tapb, ConvGeom *g, const char *what);  // abi.hip
+int conv_f16_direct(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *a, const void *b,
+                    void *out, hipStream_t s);  // conv_direct_f16.hip
 
 namespace {
 
@@ -23,7 +25,7 @@ int run_conv_f16(const unit_conv_desc *d, const ConvGeom &g0, const void *a, con
   // weight element (ko, tap, i, o): ((ko * ntaps + tap) * 16 + i) * 16 + o  -> k = tap*16 + i
   typename XL::Params xp{static_cast<const char *>(b), d->K, g.ntaps * 16, 16, (size_t)g.ntaps * 512, 32};
   typename YL::Params yp{static_cast<const char *>(a), g};
-  typename Epi::Params ep{out, d->K, g.OH * g.OW, g.npix, g.by_ohw};
+  typename Epi::Params ep{out, d->K, g.OH * g.OW, g.npix, g.by_ohw, nullptr, 1};
   const int gx = ceil_div(d->K, T::BX), gy = ceil_div(g.npix, T::BY);
   const int panel = plan.panel > 0 && plan.panel < gx ? plan.panel : 0;
   char tail[16] = "";
@@ -73,6 +75,7 @@ extern "C" int unit_conv2d_nchw16c_f16f32(const unit_conv_desc *d, const void *a
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int ntable = (int)(sizeof(kTunedF16) / sizeof(kTunedF16[0])) - 1;
   // no k-splits: fp32 atomics would make the summation order, and so the result, vary run to run
-  const ConvPlan p = plan_conv(d, g.npix, g.ntaps * 32, kTunedF16, ntable, false);
+  const ConvPlan p = plan_conv(d, g.npix, g.ntaps * 32, kTunedF16, ntable, false, true);
+  if (kConvTiles[p.variant].direct) return conv_f16_direct(p, d, g, a, b, out, s);
   return run_conv_f16_variant(p, d, g, a, b, out, s);
 }

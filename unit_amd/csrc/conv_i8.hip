@@ -18,6 +18,12 @@ const TunedConv kTunedI8[] = {
     {0, 0, 0, 0, 0, 0, 0, 0, 0},
 };
 }  // namespace
+
+// the tuned choices also serve the fused signed operator (same shapes, same kernels)
+const TunedConv *tuned_conv_i8(int *n) {
+  *n = (int)(sizeof(kTunedI8) / sizeof(kTunedI8[0])) - 1;
+  return kTunedI8;
+}
 }  // namespace unit
 
 extern "C" int unit_conv_variant_count(void) { return unit::kNumConvTiles; }
@@ -34,7 +40,7 @@ extern "C" int unit_conv2d_nchwc_u8s8s32(const unit_conv_desc *d, const void *da
   if (int rc = check_device()) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int ntable = (int)(sizeof(kTunedI8) / sizeof(kTunedI8[0])) - 1;
-  const ConvPlan p = plan_conv(d, g.npix, g.ntaps * d->cb, kTunedI8, ntable, true);
+  const ConvPlan p = plan_conv(d, g.npix, g.ntaps * d->cb, kTunedI8, ntable, true, d->cb == 16 && d->KH * d->KW <= 31);
   if (kConvTiles[p.variant].direct) return conv_i8_direct(p, d, g, data, weight, out, s);
   return d->cb == 16 ? conv_i8_c16(p, d, g, data, weight, out, s) : conv_i8_c4(p, d, g, data, weight, out, s);
 }

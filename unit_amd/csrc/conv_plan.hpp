@@ -48,11 +48,15 @@ inline ConvPlan heuristic_plan(int npix, int K, int kbytes, bool allow_split, bo
   const bool k128 = kbytes % 128 == 0;
   const auto tiles = [&](int bx, int by) { return (long)ceil_div(K, bx) * ceil_div(npix, by); };
   if (direct_ok) {
-    // int8 NCHW16c: the direct kernels won every tuned layer but the widest outputs.  One wave per
+    // NCHW16c: the direct kernels won every tuned layer but the widest outputs.  One wave per
     // 64 x 64 tile when the tiles alone fill the SIMDs, else k-groups (4, 8) to put about a
-    // thousand waves on the chip; the smallest problems use 64 x 32 tiles.
+    // thousand waves on the chip; the smallest problems use 64 x 32 (fp16: 32 x 64) tiles.
     const long t64 = tiles(64, 64);
-    const int v = t64 >= 512 ? 64 : (t64 >= 256 ? 63 : (t64 >= 96 ? 53 : 60));
+    int v;
+    if (allow_split)  // the int8 operator
+      v = t64 >= 512 ? 64 : (t64 >= 256 ? 63 : (t64 >= 96 ? 53 : 60));
+    else
+      v = t64 >= 512 ? 65 : (t64 >= 96 ? 63 : 61);
     return ConvPlan{v, 1, 0};
   }
   int v;
@@ -80,8 +84,7 @@ inline ConvPlan heuristic_plan(int npix, int K, int kbytes, bool allow_split, bo
 }
 
 inline ConvPlan plan_conv(const unit_conv_desc *d, int npix, int kbytes, const TunedConv *table, int ntable,
-                          bool allow_split) {
-  const bool direct_ok = allow_split && d->cb == 16 && d->KH * d->KW <= 31;  // allow_split: the int8 operator
+                          bool allow_split, bool direct_ok) {
   ConvPlan p = heuristic_plan(npix, d->K, kbytes, allow_split, direct_ok);
   // UNIT_AMD_CONV_NOTABLE=1: heuristic only (the tuner measures it as the baseline)
   if (tuning_override("UNIT_AMD_CONV_NOTABLE") > 0) ntable = 0;

@@ -71,6 +71,9 @@ struct ConvEpilogue {
     int ohw;   // OH * OW
     int npix;  // N * OH * OW
     FastDiv by_ohw;
+    // fused int8 form (apps/cpu/relay/result.log:17-20): out = (acc + bias[channel]) * scale
+    const int *bias;  // K values or null
+    int scale;
   };
   static constexpr int kPitch = 144;               // bytes per pixel row of the scratch
   static constexpr int kScratch = 32 * kPitch;     // per wave
@@ -92,7 +95,10 @@ struct ConvEpilogue {
     if constexpr (Op::kInt) {
       if (half == 0) {
 #pragma unroll
-        for (int i = 0; i < T::TX; ++i) wsb[i * 32 + l32] = wsx[i] << 7;
+        for (int i = 0; i < T::TX; ++i) {
+          const int c = xw0 + i * 32 + l32;
+          wsb[i * 32 + l32] = (wsx[i] << 7) + (p.bias != nullptr && c < p.K ? p.bias[c] : 0);
+        }
       }
     }
     const int ko_planes = p.K >> 4;
@@ -116,7 +122,7 @@ struct ConvEpilogue {
         for (int q = 0; q < 4; ++q) {
           const int cl = i * 32 + 8 * q + 4 * half;  // channel inside the wave's X range
           out4_t v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-          if constexpr (Op::kInt) v += *reinterpret_cast<const v4i *>(wsb + cl);
+          if constexpr (Op::kInt) v = (v + *reinterpret_cast<const v4i *>(wsb + cl)) * p.scale;
           *reinterpret_cast<out4_t *>(scratch + l32 * kPitch + (8 * q + 4 * half) * 4) = v;
         }
 #pragma unroll

@@ -127,6 +127,57 @@ def conv2d_NCHWc_int8(data, kernel, stride, padding, dilation=1, out_dtype="int3
     return out
 
 
+def conv2d_NCHWc_int8_fused(data, kernel, bias, scale, stride, padding, dilation=1, out_dtype="int32",
+                            layout="NCHW16c", out_layout="NCHW16c"):
+    """The quantized model form of the convolution,
+    fused_nn_contrib_conv2d_NCHWc_subtract_add_multiply (apps/cpu/relay/result.log:3-26,35):
+
+        out = (conv2d_NCHWc_int8(data + 128, kernel) - 128 * sum(kernel per out channel) + bias) * scale
+
+    on signed activations, in int32.
+
+    data   int8  (N, C/cb, H, W, cb), cb in {16, 4}
+    kernel int8  (K/16, C/cb, KH, KW, cb/4, 16, 4)
+    bias   int32 (K,) / any shape with K elements, or None
+    scale  Python int
+    returns int32 (N, K/16, OH, OW, 16)
+    """
+    import ctypes
+    data = _dev(data, "data", torch.int8, 5)
+    kernel = _dev(kernel, "kernel", torch.int8, 7)
+    if out_dtype != "int32":
+        raise ValueError(f"out_dtype: only 'int32' is supported, got {out_dtype!r}")
+    _layout_block(layout, "layout")
+    if _layout_block(out_layout, "out_layout") != 16:
+        raise ValueError("out_layout: the output channel block is 16 (NCHW16c)")
+    n, cc, h, w, cb = data.shape
+    ko, cc2, kh, kw, e, kb, i4 = kernel.shape
+    if cb not in (4, 16):
+        raise ValueError(f"data: channel block must be 16 or 4, got {cb}")
+    if (cc2, e, kb, i4) != (cc, cb // 4, 16, 4):
+        raise ValueError(f"kernel: shape {tuple(kernel.shape)} does not match data {tuple(data.shape)}; "
+                         f"expected (K/16, {cc}, KH, KW, {cb // 4}, 16, 4)")
+    if bias is not None:
+        if bias.dtype != torch.int32 or bias.numel() != ko * 16 or bias.device != data.device:
+            raise ValueError(f"bias: expected {ko * 16} int32 values on {data.device}")
+        bias = bias.contiguous()
+    scale = int(scale)
+    if not -2 ** 31 <= scale < 2 ** 31:
+        raise ValueError("scale: must fit int32")
+    sh, sw = _pair(stride, "stride")
+    dh, dw = _pair(dilation, "dilation")
+    pt, pl, pb, pr = _pad4(padding)
+    d = ConvDesc(n, cc * cb, h, w, ko * 16, kh, kw, sh, sw, pt, pl, pb, pr, dh, dw, cb)
+    L = _lib.load()
+    oh, ow = ctypes.c_int32(), ctypes.c_int32()
+    check(L.unit_conv_out_hw(ctypes.byref(d), ctypes.byref(oh), ctypes.byref(ow)))
+    out = torch.empty((n, ko, oh.value, ow.value, 16), dtype=torch.int32, device=data.device)
+    check(L.unit_conv2d_nchwc_s8s8s32_fused(ctypes.byref(d), data.data_ptr(), kernel.data_ptr(),
+                                            bias.data_ptr() if bias is not None else None, scale, out.data_ptr(),
+                                            _stream()))
+    return out
+
+
 def dense_dotprod(data, weight, bias=None, out_dtype="int32"):
     """u8 (M, K) x s8 packed (N/128, K/4, 128, 4) -> i32 (M, N) = data . W^T.
     A 2-D weight (N, K) is taken as the un-packed relay.nn.dense operand."""
