@@ -241,7 +241,7 @@ def main():
                     max_rel_err=f16_err, tolerance=1e-2)
 
     # ------------------------------------------------------------------ secondary legs (BASELINE configs 0, 3, 4-fp16, layouts)
-    def conv_i8_leg(shapes, batch, iters):
+    def conv_i8_leg(shapes, batch, iters, fused=False):
         rows, tot_us, tot_ops = [], 0.0, 0.0
         for i, s in enumerate(shapes):
             cb = WL.channel_block(s.C)
@@ -252,8 +252,14 @@ def main():
             o = torch.empty((batch, s.K // 16, oh, ow, 16), dtype=torch.int32, device=dev)
             desc = _lib.ConvDesc(batch, cp, s.H, s.W, s.K, s.KH, s.KW, s.stride, s.stride, s.pad, s.pad, s.pad, s.pad,
                                  1, 1, cb)
-            f = lambda: _lib.check(L.unit_conv2d_nchwc_u8s8s32(ctypes.byref(desc), d.data_ptr(), w.data_ptr(),
-                                                               o.data_ptr(), stream))
+            if fused:  # signed activations, bias and scale: the form the reference's quantized graphs run
+                d = d.view(torch.int8)
+                bias = dev_t(rng.uniform_s8((s.K,), 5000 + i).astype(np.int32) * 1000)
+                f = lambda: _lib.check(L.unit_conv2d_nchwc_s8s8s32_fused(ctypes.byref(desc), d.data_ptr(), w.data_ptr(),
+                                                                         bias.data_ptr(), 11, o.data_ptr(), stream))
+            else:
+                f = lambda: _lib.check(L.unit_conv2d_nchwc_u8s8s32(ctypes.byref(desc), d.data_ptr(), w.data_ptr(),
+                                                                   o.data_ptr(), stream))
             us = time_us(f, iters)
             ops = 2 * WL.macs(s, batch)
             rows.append(dict(layer=s.name, us=round(us, 2), tops=round(ops / us / 1e6, 2), kernel=U.last_variant()))
@@ -267,6 +273,11 @@ def main():
     single_rows, _, _ = conv_i8_leg((WL.SINGLE_CONV,), 1, 50)
     single_conv = dict(workload="N=1 C=64 56x56 K=64 3x3 s1 p1 NCHW16c (BASELINE configs[0])", **single_rows[0],
                        reference_us=24.27, reference_source="cpu-tune.log:160 (x86 VNNI, hardware unstated)")
+
+    fu_rows, fu_us, fu_ops = conv_i8_leg(WL.RESNET50, BATCH, 20, fused=True)
+    fused_s8 = dict(workload="ResNet-50 v1 conv stack, batch 32, fused signed form (conv + bias) * scale of "
+                             "apps/cpu/relay/result.log:3-26 (s8 x s8 -> i32)",
+                    stack_us=round(fu_us, 1), tops=round(fu_ops / fu_us / 1e6, 2), layers=fu_rows)
 
     # fp16 variant of the ResNet-50 b32 sweep: valid convolution on pre-padded NCHW16c inputs
     f16_rows, f16_us, f16_flops = [], 0.0, 0.0
@@ -387,6 +398,7 @@ def main():
         "single_conv": single_conv,
         "resnet18_b1": resnet18_b1,
         "conv_fp16_resnet50_b32": conv_fp16,
+        "conv_fused_s8_resnet50_b32": fused_s8,
         "layout_kernels": layout,
         "layers": table,
     }
