@@ -325,7 +325,10 @@ def main():
     # register-only MFMA throughput of this box (no memory traffic): what the silicon sustains
     sink = torch.zeros(4, dtype=torch.int32, device=dev)
     probe = {}
-    for f16, key, per in ((0, "int8_tops", 65536.0), (1, "fp16_tflops", 32768.0)):
+    # (constant operands, then operands whose bits change from one MFMA to the next: clocks follow
+    # power, and the bench data is uniform random)
+    for f16, key, per in ((0, "int8_tops", 65536.0), (1, "fp16_tflops", 32768.0),
+                          (2, "int8_tops_random_operands", 65536.0), (3, "fp16_tflops_random_operands", 32768.0)):
         blocks, iters = 512, 4000
         L.unit_mfma_peak(f16, blocks, 200, sink.data_ptr(), stream)
         us = time_us(lambda: _lib.check(L.unit_mfma_peak(f16, blocks, iters, sink.data_ptr(), stream)), 3, warm=1)

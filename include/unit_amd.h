@@ -167,6 +167,9 @@ int unit_mfma_tile_f16(const void *a, const void *b, void *c, unit_stream_t stre
  * 4 * iters MFMAs per wavefront (int8 32x32x32 when f16 == 0, else fp16 32x32x16) on 4
  * independent accumulator chains with no memory traffic.  Operations issued =
  * blocks * 4 * 4 * iters * 65536 (int8) or * 32768 (fp16); the caller times the launch.
+ * `f16` bit 1 (values 2, 3) selects operands with random bit patterns that change from one
+ * instruction to the next instead of constant ones: the chip's clocks follow its power draw, and
+ * the rate it sustains depends on how many operand bits toggle.
  * `sink` is a 4-byte device scratch word. */
 int unit_mfma_peak(int32_t f16, int32_t blocks, int32_t iters, void *sink, unit_stream_t stream);
 

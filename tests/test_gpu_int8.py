@@ -55,6 +55,19 @@ def test_dense_bit_exact(dev, oracle, M, N, K, packed):
     assert np.array_equal(out.cpu().numpy(), ref), U.last_variant()
 
 
+@pytest.mark.parametrize("M,N,K", [(300, 384, 272), (37, 256, 16), (512, 640, 400), (1, 128, 48)])
+def test_dense_packed_weights_direct_to_registers(dev, oracle, monkeypatch, M, N, K):
+    """The kernel variant that reads the pre-packed weight straight into MFMA fragments, forced on
+    ragged shapes: M and N tile edges, a K tail of 16 .. 112 bytes, one k-step."""
+    monkeypatch.setenv("UNIT_AMD_DENSE_VARIANT", "13")
+    a = rng.uniform_u8((M, K), 300 + M)
+    wp = oracle.prepack_dense_weight(rng.uniform_s8((N, K), 400 + N))
+    out = U.dense_dotprod(_t(a, dev), _t(wp, dev))
+    torch.cuda.synchronize()
+    assert "direct" in U.last_variant()
+    assert np.array_equal(out.cpu().numpy(), oracle.c_dense(a, wp)), U.last_variant()
+
+
 def test_dense_extremes(dev, oracle):
     """255 x -128 everywhere: the largest negative accumulation (K * -32640), and 255 x 127."""
     M, N, K = 64, 128, 4096

@@ -113,21 +113,35 @@ __global__ __launch_bounds__(64) void mfma_tile_f16(const char *a, const char *b
 
 // Register-only MFMA throughput probe in the manner of poc/vnni/micro.cc:16-51: 4 independent
 // accumulator chains per wave, no memory traffic; one workgroup of 4 waves per launch slot.
-template <class Op>
+// RANDOM: four operand pairs of hashed bits, rotated so that consecutive MFMAs see different data
+template <class Op, bool RANDOM>
 __global__ __launch_bounds__(256) void mfma_peak(int iters, typename Op::out_t *sink) {
   const int l = threadIdx.x;
-  v4i x = {l, l + 1, l + 2, l + 3}, y = {l ^ 5, l ^ 9, l ^ 3, l ^ 7};
-  if (!Op::kInt) {
-    x = v4i{0x3c003c00, 0x3c003c00, 0x3c003c00, 0x3c003c00};
-    y = x;
+  v4i xs[4], ys[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    xs[i] = v4i{l, l + 1, l + 2, l + 3};
+    ys[i] = v4i{l ^ 5, l ^ 9, l ^ 3, l ^ 7};
+    if (!Op::kInt) xs[i] = ys[i] = v4i{0x3c003c00, 0x3c003c00, 0x3c003c00, 0x3c003c00};
+    if (RANDOM) {
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        u32 h = (u32)(l * 32 + i * 8 + d) * 2654435761u;
+        h ^= h >> 15; h *= 2246822519u; h ^= h >> 13; h *= 3266489917u; h ^= h >> 16;
+        u32 g = h * 2654435761u + 0x9e3779b9u;
+        g ^= g >> 15; g *= 2246822519u; g ^= g >> 13;
+        xs[i][d] = (int)(Op::kInt ? h : (h & 0x3fff3fffu));  // fp16: finite values below 2
+        ys[i][d] = (int)(Op::kInt ? g : (g & 0x3fff3fffu));
+      }
+    }
   }
   typename Op::acc_t a0, a1, a2, a3;
   for (int r = 0; r < 16; ++r) a0[r] = a1[r] = a2[r] = a3[r] = 0;
   for (int i = 0; i < iters; ++i) {
-    a0 = Op::mma(x, y, a0);
-    a1 = Op::mma(x, y, a1);
-    a2 = Op::mma(x, y, a2);
-    a3 = Op::mma(x, y, a3);
+    a0 = Op::mma(xs[0], ys[1], a0);
+    a1 = Op::mma(xs[1], ys[2], a1);
+    a2 = Op::mma(xs[2], ys[3], a2);
+    a3 = Op::mma(xs[3], ys[0], a3);
   }
   typename Op::out_t s = 0;
   for (int r = 0; r < 16; ++r) s += a0[r] + a1[r] + a2[r] + a3[r];
@@ -142,10 +156,12 @@ extern "C" int unit_mfma_peak(int32_t f16, int32_t blocks, int32_t iters, void *
   if (!sink || blocks <= 0 || iters <= 0) return fail(UNIT_E_ARG, "unit_mfma_peak: bad arguments");
   if (int rc = check_device()) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (f16)
-    hipLaunchKernelGGL(mfma_peak<OpF16>, dim3(blocks), dim3(256), 0, s, iters, static_cast<float *>(sink));
-  else
-    hipLaunchKernelGGL(mfma_peak<OpI8>, dim3(blocks), dim3(256), 0, s, iters, static_cast<int *>(sink));
+  switch (f16 & 3) {
+    case 0: hipLaunchKernelGGL((mfma_peak<OpI8, false>), dim3(blocks), dim3(256), 0, s, iters, static_cast<int *>(sink)); break;
+    case 1: hipLaunchKernelGGL((mfma_peak<OpF16, false>), dim3(blocks), dim3(256), 0, s, iters, static_cast<float *>(sink)); break;
+    case 2: hipLaunchKernelGGL((mfma_peak<OpI8, true>), dim3(blocks), dim3(256), 0, s, iters, static_cast<int *>(sink)); break;
+    default: hipLaunchKernelGGL((mfma_peak<OpF16, true>), dim3(blocks), dim3(256), 0, s, iters, static_cast<float *>(sink)); break;
+  }
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "unit_mfma_peak: %s", hipGetErrorString(e));
 }

@@ -3,6 +3,7 @@
 #include "epilogues.hpp"
 #include "host.hpp"
 #include "loaders.hpp"
+#include "gemm_mixed.hpp"
 #include "mma_dma.hpp"
 
 namespace unit {
@@ -60,6 +61,33 @@ int run_dense_dma(const void *a, const void *w, void *c, int M, int N, int K, hi
   return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "unit_dense_u8s8s32: launch: %s", hipGetErrorString(e));
 }
 
+// pre-packed weights straight to registers, activations through LDS (UNIT_AMD_DENSE_VARIANT=13).
+// Measured equal to the staged kernel (91.6 vs 91.1 us at 4096^3) although it moves 1.6 x less
+// through LDS: the GEMM is bound by instruction issue per SIMD, not by the LDS pipe.
+int run_dense_mixed(const void *a, const void *wp, void *c, int M, int N, int K, hipStream_t s) {
+  using T = Tile<256, 256, 128, 2, 4>;
+  using XL = RowMajorLoader<T::BX, T::BKB, T::NT, true>;
+  using Epi = GemmEpilogue<OpI8, false>;
+  const char *what = "unit_dense_dotprod_u8s8s32";
+  typename XL::Params xp{static_cast<const char *>(a), M, K, K};
+  typename Epi::Params ep{c, M, N};
+  const int nk = ceil_div(K, T::BKB), gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
+  constexpr int lds = 2 * T::XBYTES;
+  auto kern = gemm_mixed_i8<T>;
+  static thread_local bool allowed = false;
+  if (!allowed) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
+    if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "%s: hipFuncSetAttribute: %s", what, hipGetErrorString(e));
+    allowed = true;
+  }
+  GridMap gm{gx, gy, gx < 4 ? gx : 4, 1, gx * gy};
+  set_variant("i8densepk_direct_x%d_y%d_k%d_w%d_s1", T::BX, T::BY, T::BKB, T::NT / 64);
+  hipLaunchKernelGGL(kern, dim3(gm.total), dim3(T::NT), lds, s, xp, static_cast<const char *>(wp), N, K / 4, ep, nk, gm);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "%s: launch: %s", what, hipGetErrorString(e));
+}
+
 template <bool PACKED>
 int dense(const void *a, const void *w, void *c, int M, int N, int K, unit_stream_t stream) {
   const char *what = PACKED ? "unit_dense_dotprod_u8s8s32" : "unit_dense_u8s8s32";
@@ -86,6 +114,8 @@ int dense(const void *a, const void *w, void *c, int M, int N, int K, unit_strea
     case 10: if (!PACKED && K % 64 == 0) return run_dense_dma<Tile<256, 256, 64, 2, 2>, 3>(a, w, c, M, N, K, s); break;
     case 11: if (!PACKED && K % 64 == 0) return run_dense_dma<Tile<256, 128, 64, 2, 2>, 4>(a, w, c, M, N, K, s); break;
     case 12: if (!PACKED && K % 128 == 0) return run_dense_dma<Tile<256, 256, 128, 2, 4>, 2>(a, w, c, M, N, K, s); break;
+    case 13: if (PACKED) return run_dense_mixed(a, w, c, M, N, K, s); break;
+    case 14: return run_dense<Tile<256, 256, 128, 2, 4>, PACKED>(a, w, c, M, N, K, s);
     default: break;
   }
   if (M >= 256 && N >= 256 && tiles_big >= 128) return run_dense<Tile<256, 256, 128, 2, 4>, PACKED>(a, w, c, M, N, K, s);
