@@ -279,6 +279,25 @@ def main():
                              "apps/cpu/relay/result.log:3-26 (s8 x s8 -> i32)",
                     stack_us=round(fu_us, 1), tops=round(fu_ops / fu_us / 1e6, 2), layers=fu_rows)
 
+    # 3-D convolution workloads of apps/cpu/kernel/conv3d.py:13-25 (depth 16, batch 1; the 4-channel one left out)
+    c3_rows = []
+    for i, (ic, h, w_, oc, ks, st) in enumerate(((256, 16, 16, 256, 3, 1), (512, 9, 9, 512, 3, 1), (128, 30, 30, 128, 3, 1),
+                                                   (64, 56, 56, 128, 1, 2), (64, 58, 58, 64, 3, 1), (128, 28, 28, 256, 1, 2),
+                                                   (256, 16, 16, 512, 3, 2), (64, 58, 58, 128, 3, 2), (128, 30, 30, 256, 3, 2),
+                                                   (256, 14, 14, 512, 1, 2))):
+        a3 = torch.randint(-128, 128, (1, ic // 16, 16, h, w_, 16), dtype=torch.int8, device=dev)
+        w3 = torch.randint(-128, 128, (oc // 16, ic // 16, ks, ks, ks, 4, 16, 4), dtype=torch.int8, device=dev)
+        od, oh, ow = (16 - ks) // st + 1, (h - ks) // st + 1, (w_ - ks) // st + 1
+        o3 = torch.empty((1, oc // 16, od, oh, ow, 16), dtype=torch.int32, device=dev)
+        d3 = _lib.Conv3dDesc(1, ic, 16, h, w_, oc, ks, ks, ks, st)
+        f = lambda: _lib.check(L.unit_conv3d_ncdhwc_s8s8s32(ctypes.byref(d3), a3.data_ptr(), w3.data_ptr(), o3.data_ptr(),
+                                                            stream))
+        us = time_us(f, 20)
+        ops = 2.0 * od * oh * ow * oc * ic * ks ** 3
+        c3_rows.append(dict(workload=f"{ic}x16x{h}x{w_} -> {oc}, {ks}^3 s{st}", us=round(us, 2),
+                            tops=round(ops / us / 1e6, 1), kernel=U.last_variant()))
+    conv3d = dict(workload="3-D int8 convolutions of apps/cpu/kernel/conv3d.py:13-25, NCDHW16c, s8 x s8 -> i32", layers=c3_rows)
+
     # fp16 variant of the ResNet-50 b32 sweep: valid convolution on pre-padded NCHW16c inputs
     f16_rows, f16_us, f16_flops = [], 0.0, 0.0
     for i, s in enumerate(WL.RESNET50):
@@ -402,6 +421,7 @@ def main():
         "resnet18_b1": resnet18_b1,
         "conv_fp16_resnet50_b32": conv_fp16,
         "conv_fused_s8_resnet50_b32": fused_s8,
+        "conv3d_s8": conv3d,
         "layout_kernels": layout,
         "layers": table,
     }

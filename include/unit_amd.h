@@ -88,6 +88,22 @@ int unit_conv2d_nchwc_u8s8s32(const unit_conv_desc *d, const void *data, const v
 int unit_conv2d_nchwc_s8s8s32_fused(const unit_conv_desc *d, const void *data, const void *weight,
                                     const int32_t *bias, int32_t scale, void *out, unit_stream_t stream);
 
+/* 3-D convolution of apps/cpu/kernel/conv3d.py:39-64 (the reference's only closed form of the
+ * blocked convolution): valid (no padding), one stride for the three dimensions, s8 x s8 -> i32
+ * as its te.compute casts both operands from int8:
+ *   O[n,ko,x,y,z,kb] = sum_{ci,rd,rh,rw,e,i} A[n,ci,s*x+rd,s*y+rh,s*z+rw,4e+i] * W[ko,ci,rd,rh,rw,e,kb,i]
+ *   data   s8  (N, C/16, D, H, W, 16)
+ *   weight s8  (K/16, C/16, KD, KH, KW, 4, 16, 4)
+ *   out    i32 (N, K/16, OD, OH, OW, 16),  O* = (* - K*) / stride + 1
+ * 16-channel blocks only (the 4-channel 7x7x7 workload of conv3d.py:22 is not covered). */
+typedef struct unit_conv3d_desc {
+  int32_t N, C, D, H, W; /* data: batch, input channels (multiple of 16), depth, height, width */
+  int32_t K, KD, KH, KW; /* output channels (multiple of 16), kernel depth, height, width */
+  int32_t stride;
+} unit_conv3d_desc;
+int unit_conv3d_ncdhwc_s8s8s32(const unit_conv3d_desc *d, const void *data, const void *weight, void *out,
+                               unit_stream_t stream);
+
 /* topi.x86.dense_dotprod(data, weight, None, 'int32') as called at
  * apps/cpu/kernel/int8-gemm.py:13-16.
  *   a   u8  (M, K) row-major

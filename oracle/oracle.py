@@ -233,6 +233,32 @@ def conv2d_nchwc_int8_fused(data_s8, weight, bias, scale, stride=1, padding=0, d
     return np.ascontiguousarray((out & 0xFFFFFFFF).astype(np.uint32).view(np.int32))
 
 
+def conv3d_ncdhwc_int8(data, weight, stride=1):
+    """apps/cpu/kernel/conv3d.py:39-64, the reference's own te.compute: valid 3-D convolution, one
+    stride, both operands int8 cast to int32:
+
+    O[n,ko,x,y,z,kb] = sum_{rco,rd,rh,rw,rcm,rci} A[n,rco,s*x+rd,s*y+rh,s*z+rw,4*rcm+rci] * B[ko,rco,rd,rh,rw,rcm,kb,rci]
+    """
+    data = np.asarray(data)
+    weight = np.asarray(weight)
+    assert data.dtype == np.int8 and weight.dtype == np.int8
+    n, cc, dd, h, w, cb = data.shape
+    ko, cc2, kd, kh, kw, e, kb, i4 = weight.shape
+    assert cc == cc2 and kb == 16 and i4 == 4 and e * 4 == cb
+    s = int(stride)
+    od, oh, ow = (dd - kd) // s + 1, (h - kh) // s + 1, (w - kw) // s + 1
+    a = data.astype(np.int64)
+    wt = weight.astype(np.int64).transpose(0, 6, 1, 2, 3, 4, 5, 7).reshape(ko * 16, cc, kd, kh, kw, cb)
+    out = np.zeros((n, ko * 16, od, oh, ow), dtype=np.int64)
+    for z in range(kd):
+        for y in range(kh):
+            for x in range(kw):
+                win = a[:, :, z:z + (od - 1) * s + 1:s, y:y + (oh - 1) * s + 1:s, x:x + (ow - 1) * s + 1:s, :]
+                out += np.einsum("ncdhwi,kci->nkdhw", win, wt[:, :, z, y, x, :], optimize=True)
+    out = out.reshape(n, ko, 16, od, oh, ow).transpose(0, 1, 3, 4, 5, 2)
+    return np.ascontiguousarray((out & 0xFFFFFFFF).astype(np.uint32).view(np.int32))
+
+
 # --------------------------------------------------------------------------- a3 dense
 def dense_logical(a, w):
     """relay.nn.dense(x, w) of apps/cpu/relay/int8-gemm.py:14-16: C = A . W^T, A u8 (M,K), W s8 (N,K)."""

@@ -198,6 +198,45 @@ def test_conv2d_fused_every_direct_variant(dev, oracle, monkeypatch):
     assert len(names) >= 15 and all(n.startswith("s8direct") for n in names)
 
 
+CONV3D_CASES = [
+    # C, D, H, W, K, kernel, stride: apps/cpu/kernel/conv3d.py:13-25 (d = 16 there; depth cut where the oracle would take minutes)
+    (256, 16, 16, 16, 256, 3, 1),
+    (512, 16, 9, 9, 512, 3, 1),
+    (128, 6, 30, 30, 128, 3, 1),
+    (64, 16, 56, 56, 128, 1, 2),
+    (64, 5, 58, 58, 64, 3, 1),
+    (256, 16, 16, 16, 512, 3, 2),
+    (256, 16, 14, 14, 512, 1, 2),
+    (16, 4, 7, 9, 32, 3, 1),      # 27 taps: odd, the last k-step is half padding; ragged pixel count
+    (48, 3, 5, 5, 16, (1, 3, 2), 1),
+]
+
+
+@pytest.mark.parametrize("C,D,H,W,K,ks,stride", CONV3D_CASES)
+def test_conv3d_bit_exact(dev, oracle, C, D, H, W, K, ks, stride):
+    kd, kh, kw = (ks,) * 3 if isinstance(ks, int) else ks
+    x = rng.uniform_s8((1, C // 16, D, H, W, 16), 17 * C + H)
+    wt = rng.uniform_s8((K // 16, C // 16, kd, kh, kw, 4, 16, 4), 19 * K + kd)
+    ref = oracle.conv3d_ncdhwc_int8(x, wt, stride)
+    out = U.conv3d_NCDHWc_int8(_t(x, dev), _t(wt, dev), stride)
+    torch.cuda.synchronize()
+    assert tuple(out.shape) == ref.shape
+    assert np.array_equal(out.cpu().numpy(), ref), U.last_variant()
+
+
+def test_conv3d_every_direct_variant(dev, oracle, monkeypatch):
+    from unit_amd import _lib
+    x = rng.uniform_s8((2, 3, 5, 7, 9, 16), 23)
+    wt = rng.uniform_s8((5, 3, 3, 3, 3, 4, 16, 4), 29)
+    ref = oracle.conv3d_ncdhwc_int8(x, wt, 1)
+    tx, tw = _t(x, dev), _t(wt, dev)
+    for v in range(1, _lib.load().unit_conv_variant_count() + 1):
+        monkeypatch.setenv("UNIT_AMD_CONV_VARIANT", str(v))
+        out = U.conv3d_NCDHWc_int8(tx, tw, 1)
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy(), ref), (v, U.last_variant())
+
+
 def test_conv2d_zero_padding_value(dev, oracle):
     """Padded pixels are u8 zeros: with all-255 data and all-ones weights every output equals
     255 * (number of in-image taps) * C, which differs between border and interior."""

@@ -18,6 +18,7 @@ SYMBOLS = (
     "unit_conv_out_hw",
     "unit_conv2d_nchwc_u8s8s32",
     "unit_conv2d_nchwc_s8s8s32_fused",
+    "unit_conv3d_ncdhwc_s8s8s32",
     "unit_dense_dotprod_u8s8s32",
     "unit_dense_u8s8s32",
     "unit_gemm_f16",
@@ -37,6 +38,11 @@ class ConvDesc(ctypes.Structure):
     """struct unit_conv_desc"""
     _fields_ = [(k, ctypes.c_int32) for k in
                 ("N", "C", "H", "W", "K", "KH", "KW", "sh", "sw", "pt", "pl", "pb", "pr", "dh", "dw", "cb")]
+
+
+class Conv3dDesc(ctypes.Structure):
+    """struct unit_conv3d_desc"""
+    _fields_ = [(k, ctypes.c_int32) for k in ("N", "C", "D", "H", "W", "K", "KD", "KH", "KW", "stride")]
 
 
 class UnitError(RuntimeError):
@@ -64,6 +70,7 @@ def load():
     L.unit_conv_out_hw.argtypes = [dp, ctypes.POINTER(i32), ctypes.POINTER(i32)]
     L.unit_conv2d_nchwc_u8s8s32.argtypes = [dp, vp, vp, vp, vp]
     L.unit_conv2d_nchwc_s8s8s32_fused.argtypes = [dp, vp, vp, vp, i32, vp, vp]
+    L.unit_conv3d_ncdhwc_s8s8s32.argtypes = [ctypes.POINTER(Conv3dDesc), vp, vp, vp, vp]
     L.unit_dense_dotprod_u8s8s32.argtypes = [vp, vp, vp, i32, i32, i32, vp]
     L.unit_dense_u8s8s32.argtypes = [vp, vp, vp, i32, i32, i32, vp]
     L.unit_gemm_f16.argtypes = [vp, vp, vp, i32, i32, i32, i32, vp]

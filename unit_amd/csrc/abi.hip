@@ -85,6 +85,10 @@ int conv_geom(const unit_conv_desc *d, int tapb, ConvGeom *g, const char *what) 
   g->by_ow = FastDiv::make(OW);
   g->by_kh = FastDiv::make(d->KH);
   g->by_kw = FastDiv::make(d->KW);
+  g->D = g->KD = g->sd = 1;
+  g->nopad = !(d->pt || d->pl || d->pb || d->pr);
+  g->by_plane = g->by_ohw;
+  g->by_kd = FastDiv::make(1);
   return UNIT_OK;
 }
 

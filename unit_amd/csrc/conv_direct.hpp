@@ -106,19 +106,20 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
   int *wsum = reinterpret_cast<int *>(lds + S::template lds_fixed<Op>() - S::WSUM);
   v2i *tab = reinterpret_cast<v2i *>(lds + S::template lds_fixed<Op>());
 
-  // tap -> (byte offset of the tap inside an image relative to the window origin, index of its
-  // window position kh * KW + kw).  int8 pairs taps into k-steps: the odd tap past the end points
+  // tap (ci, kd, kh, kw) -> (byte offset of the tap inside an image relative to the window origin,
+  // index of its window position kh * KW + kw).  int8 pairs taps into k-steps: the odd tap past the end points
   // at bit 31 of the window set, which is never set, so it is staged like zero padding.
   const int nsteps = kInt ? (g.ntaps + 1) >> 1 : g.ntaps;
   const int ntab = kInt ? 2 * nsteps : nsteps;
   for (int e = threadIdx.x; e < ntab; e += S::NT) {
     v2i ent = {0, 31};
     if (e < g.ntaps) {
-      int kw, rest, kh, ci;
+      int kw, rest, kh, rest2, kd, ci;
       g.by_kw.divmod(e, rest, kw);
-      g.by_kh.divmod(rest, ci, kh);
-      ent[0] = ((ci * g.H + kh * g.dh) * g.W + kw * g.dw) * TAPB;
-      ent[1] = kh * g.KW + kw;
+      g.by_kh.divmod(rest, rest2, kh);
+      g.by_kd.divmod(rest2, ci, kd);
+      ent[0] = (((ci * g.D + kd) * g.H + kh * g.dh) * g.W + kw * g.dw) * TAPB;
+      ent[1] = g.nopad ? 0 : kh * g.KW + kw;
     }
     tab[e] = ent;
   }
@@ -150,17 +151,18 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
     pixoff[j] = kInt ? 0 : half * 16;
     inside[j] = 0;
     if (m < g.npix) {
-      int n, rem, oh, ow;
+      int n, rem, od, rem2, oh, ow;
       g.by_ohw.divmod(m, n, rem);
-      g.by_ow.divmod(rem, oh, ow);
+      g.by_plane.divmod(rem, od, rem2);  // od = 0 for a 2-D convolution
+      g.by_ow.divmod(rem2, oh, ow);
       const int ih0 = oh * g.sh - g.pt, iw0 = ow * g.sw - g.pl;
-      pixoff[j] += (int)(n * g.img_bytes) + (ih0 * g.W + iw0) * TAPB;
+      pixoff[j] += (int)(n * g.img_bytes) + ((od * g.sd * g.H + ih0) * g.W + iw0) * TAPB;
       if constexpr (S::PAD) {
         u32 cols = 0, bits = 0;  // columns kw inside the image; then one copy of them per row kh inside
         for (int kw = 0; kw < g.KW; ++kw) cols |= (u32)((u32)(iw0 + kw * g.dw) < (u32)g.W) << kw;
         for (int kh = 0; kh < g.KH; ++kh)
           if ((u32)(ih0 + kh * g.dh) < (u32)g.H) bits |= cols << (kh * g.KW);
-        inside[j] = bits;
+        inside[j] = g.nopad ? 1u : bits;  // without padding every real tap carries position 0
       }
     }
   }

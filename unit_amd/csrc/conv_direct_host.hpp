@@ -19,7 +19,7 @@ int run_direct(const char *what, const char *tag, const unit_conv_desc *d, const
     if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "%s: hipFuncSetAttribute: %s", what, hipGetErrorString(e));
     lds_allowed = kMaxLds;
   }
-  typename ConvEpilogue<Op>::Params ep{out, d->K, g.OH * g.OW, g.npix, g.by_ohw, bias, scale};
+  typename ConvEpilogue<Op>::Params ep{out, d->K, g.by_ohw.d, g.npix, g.by_ohw, bias, scale};
   GridMap gm;
   gm.gx = ceil_div(d->K, S::BX);
   gm.gy = ceil_div(g.npix, S::BY);

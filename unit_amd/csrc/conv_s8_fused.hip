@@ -11,14 +11,11 @@ namespace unit {
 int conv_geom(const unit_conv_desc *d, int tapb, ConvGeom *g, const char *what);  // abi.hip
 const TunedConv *tuned_conv_i8(int *n);                                             // conv_i8.hip
 
-namespace {
-
-const char *kWhat = "unit_conv2d_nchwc_s8s8s32_fused";
-
-int direct_s8(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
-              const int *bias, int scale, void *out, hipStream_t s) {
+// direct kernels on signed data; `what` names the entry point in messages (also used by the 3-D operator)
+int conv_s8_direct(const char *kWhat, const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data,
+                   const void *w, const int *bias, int scale, void *out, hipStream_t s) {
   // an odd tap count needs the tap masks for the tap that pads the last k-step
-  const bool masked = d->pt || d->pl || d->pb || d->pr || (g.ntaps & 1);
+  const bool masked = !g.nopad || (g.ntaps & 1);
 #define UNIT_CONV_VARIANT(ID, BX, BY, BKB, WX, WY, PF, FF, KG)
 #define UNIT_CONV_DIRECT(ID, TX, TY, KG, D)                                                                          \
   case ID:                                                                                                           \
@@ -34,6 +31,10 @@ int direct_s8(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, 
 #undef UNIT_CONV_DIRECT
 #undef UNIT_CONV_VARIANT
 }
+
+namespace {
+
+const char *kWhat = "unit_conv2d_nchwc_s8s8s32_fused";
 
 template <int TAPB>
 int staged_s8(const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w, const int *bias, int scale,
@@ -65,7 +66,7 @@ extern "C" int unit_conv2d_nchwc_s8s8s32_fused(const unit_conv_desc *d, const vo
     ConvPlan p = plan_conv(d, g.npix, g.ntaps * 16, table, ntable, true, true);
     if (!kConvTiles[p.variant].direct) p = heuristic_plan(g.npix, d->K, g.ntaps * 16, true, true);
     p.splits = 1;
-    return direct_s8(p, d, g, data, weight, bias, scale, out, s);
+    return conv_s8_direct(kWhat, p, d, g, data, weight, bias, scale, out, s);
   }
   return d->cb == 16 ? staged_s8<16>(d, g, data, weight, bias, scale, out, s)
                      : staged_s8<4>(d, g, data, weight, bias, scale, out, s);

@@ -237,7 +237,11 @@ struct ConvGeom {
   int ntaps;   // (C / cb) * KH * KW
   int ntab;    // table entries (ntaps rounded up to whole pipeline stages)
   u32 img_bytes;  // bytes per image
-  FastDiv by_ohw, by_ow, by_kh, by_kw;  // dividers by OH * OW, OW, KH, KW
+  FastDiv by_ohw, by_ow, by_kh, by_kw;  // dividers by output pixels per image, OW, KH, KW
+  // depth, for the 3-D convolution (direct kernels only); 1 / 1 / 1 / 1 for 2-D, where
+  // by_plane = by_ohw
+  int D, KD, sd, nopad;                 // nopad: no zero padding anywhere (every tap of a valid pixel is inside)
+  FastDiv by_plane, by_kd;              // dividers by OH * OW, KD
 };
 
 template <int ROWS, int BKB, int NT, int TAPB, bool XOR80, int PF = 1>
