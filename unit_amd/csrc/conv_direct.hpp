@@ -37,14 +37,21 @@ struct DirectShape {
   static constexpr bool PAD = PAD_;
   static constexpr int BX = TX * 32, BY = TY * 32;
   static constexpr int NT = 64 * KG;
-  static constexpr int kScratch = 32 * 144;       // per-wave transpose area (32 pixels x 144-byte pitch)
+  static constexpr int kScratch = 32 * 144 + 128;  // per wave: transpose area (32 pixels x 144-byte pitch) + 32 addends
   static constexpr int TILE = TX * TY * 4096;     // one 4-byte accumulator tile
   static constexpr int WSUM = TX * 32 * 4;        // summed 128 * weight sums
-  // integer partial tiles are added into one LDS tile with atomics (exact in any order); float
-  // ones are kept apart, one per wave, and summed in wave order so that results do not vary
+  // Integer partial tiles are added into one LDS tile with atomics (exact in any order).  Float
+  // ones are parked side by side and the owner of a block adds them in wave order, so that results
+  // do not vary from run to run.  (Parking integer tiles too was measured: fewer LDS instructions,
+  // but KG tiles of LDS per workgroup leave room for one workgroup per CU, and layers with 1.5
+  // tiles per CU lost 25 %.)
   template <class Op>
-  static constexpr int lds_fixed() {
-    return KG * kScratch + (KG > 1 ? (Op::kInt ? TILE : KG * TILE) : 0) + WSUM;  // the tap table follows
+  static constexpr bool parked() {
+    return !Op::kInt;
+  }
+  template <class Op>
+  static constexpr int lds_fixed() {  // the tap table follows
+    return KG * kScratch + (KG > 1 ? (parked<Op>() ? KG * (TILE + WSUM) : TILE + WSUM) : WSUM);
   }
   static_assert(NT <= 1024 && D >= 2 && D <= 8, "direct conv shape");
 };
@@ -103,7 +110,9 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
 
   char *scratch = lds + wave * S::kScratch;
   char *tiles = lds + KG * S::kScratch;
-  int *wsum = reinterpret_cast<int *>(lds + S::template lds_fixed<Op>() - S::WSUM);
+  constexpr bool kParked = KG > 1 && S::template parked<Op>();
+  // the per-channel addends: one row, or one per wave when the tiles are parked
+  int *wsum = reinterpret_cast<int *>(lds + S::template lds_fixed<Op>() - (kParked ? KG : 1) * S::WSUM);
   v2i *tab = reinterpret_cast<v2i *>(lds + S::template lds_fixed<Op>());
 
   // tap (ci, kd, kh, kw) -> (byte offset of the tap inside an image relative to the window origin,
@@ -123,9 +132,9 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
     }
     tab[e] = ent;
   }
-  if constexpr (kInt && KG > 1) {
-    int *z = reinterpret_cast<int *>(tiles);
-    for (int e = threadIdx.x; e < (S::TILE + S::WSUM) / 4; e += S::NT) z[e] = 0;
+  if constexpr (KG > 1 && !kParked) {
+    v4i *z = reinterpret_cast<v4i *>(tiles);
+    for (int e = threadIdx.x; e < (S::TILE + S::WSUM) / 16; e += S::NT) z[e] = v4i{0, 0, 0, 0};
   }
 
   int bx, by, split;
@@ -330,7 +339,7 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
       for (int j = 0; j < TY; ++j)
         store_block<Op>(ep, acc[i][j], addend ? wsum + i * 32 : nullptr, ep.scale, x0 + i * 32, y0 + j * 32, lane,
                         scratch);
-  } else if constexpr (kInt) {
+  } else if constexpr (!kParked) {
     // sum the partial tiles of the KG waves in LDS, then share the blocks among the waves
     int *sum = reinterpret_cast<int *>(tiles);
 #pragma unroll
@@ -355,16 +364,23 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
       store_block<Op>(ep, total, addend ? wsum + i * 32 : nullptr, ep.scale, x0 + i * 32, y0 + j * 32, lane, scratch);
     }
   } else {
-    // float: every wave parks its partial tile; the owner of a block adds them in wave order
-    float *mine = reinterpret_cast<float *>(tiles + wave * S::TILE);
+    // every wave parks its partial tile (and addends); the owner of a block adds them in wave order
+    using out4_t = typename Op::out4_t;
+    char *mine = tiles + wave * S::TILE;
 #pragma unroll
     for (int i = 0; i < TX; ++i)
 #pragma unroll
       for (int j = 0; j < TY; ++j)
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-          *reinterpret_cast<v4f *>(mine + (((i * TY + j) * 4 + q) * 64 + lane) * 4) =
-              v4f{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+          *reinterpret_cast<out4_t *>(mine + (((i * TY + j) * 4 + q) * 64 + lane) * 16) =
+              out4_t{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+    if constexpr (kInt) {
+      if (addend && half == 0) {
+#pragma unroll
+        for (int i = 0; i < TX; ++i) wsum[wave * (TX * 32) + i * 32 + l32] = wsx[i];
+      }
+    }
     __syncthreads();
     for (int b = wave; b < TX * TY; b += KG) {
       const int i = b / TY, j = b - i * TY;
@@ -372,15 +388,26 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
 #pragma unroll
       for (int r = 0; r < 16; ++r) total[r] = 0;
       for (int w = 0; w < KG; ++w) {
-        const float *its = reinterpret_cast<const float *>(tiles + w * S::TILE);
+        const char *its = tiles + w * S::TILE;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const v4f v = *reinterpret_cast<const v4f *>(its + ((b * 4 + q) * 64 + lane) * 4);
+          const out4_t v = *reinterpret_cast<const out4_t *>(its + ((b * 4 + q) * 64 + lane) * 16);
 #pragma unroll
           for (int e = 0; e < 4; ++e) total[4 * q + e] += v[e];
         }
       }
-      store_block<Op>(ep, total, nullptr, 1, x0 + i * 32, y0 + j * 32, lane, scratch);
+      if constexpr (kInt) {
+        // the block's addends of all waves, summed into row 0 by the lanes that hold them
+        if (addend && half == 0) {
+          int a = 0;
+          for (int w = 0; w < KG; ++w) a += wsum[w * (TX * 32) + i * 32 + l32];
+          reinterpret_cast<int *>(scratch)[1152 + l32] = a;  // behind the transpose area
+        }
+        store_block<Op>(ep, total, addend ? reinterpret_cast<const int *>(scratch) + 1152 : nullptr, ep.scale,
+                        x0 + i * 32, y0 + j * 32, lane, scratch);
+      } else {
+        store_block<Op>(ep, total, nullptr, 1, x0 + i * 32, y0 + j * 32, lane, scratch);
+      }
     }
   }
 }
