@@ -7,23 +7,34 @@
 namespace unit {
 namespace {
 
-template <class T, bool OUT_F16>
+template <class T, bool OUT_F16, int PF = 1>
 int run_gemm_f16(const void *a, const void *b, void *c, int M, int N, int K, hipStream_t s) {
-  using XL = RowMajorLoader<T::BX, T::BKB, T::NT, false>;
-  using YL = KMajorF16Loader<T::BY, T::BKB, T::NT>;
+  using XL = RowMajorLoader<T::BX, T::BKB, T::NT, false, PF>;
+  using YL = KMajorF16Loader<T::BY, T::BKB, T::NT, PF>;
   using Epi = GemmEpilogue<OpF16, OUT_F16>;
   typename XL::Params xp{static_cast<const char *>(a), M, K * 2, K * 2};
   typename YL::Params yp{static_cast<const char *>(b), N, K, N + 4, 0, N * 2};
   typename Epi::Params ep{c, M, N};
   const int nk = ceil_div(K * 2, T::BKB), gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
-  set_variant("f16gemm_x%d_y%d_k%d_w%d%s", T::BX, T::BY, T::BKB, T::NT / 64, OUT_F16 ? "_h" : "");
+  set_variant("f16gemm_x%d_y%d_k%d_w%dx%d_p%d%s", T::BX, T::BY, T::BKB, T::WX, T::WY, PF, OUT_F16 ? "_h" : "");
   return launch_mma<OpF16, T, XL, YL, Epi, WS_NONE>(xp, yp, ep, nk, gx, gy, 4, 1, c, 0, 0, s, "unit_gemm_f16");
 }
 
 template <bool OUT_F16>
 int gemm_f16(const void *a, const void *b, void *c, int M, int N, int K, hipStream_t s) {
   const long tiles_big = (long)ceil_div(M, 256) * ceil_div(N, 256);
-  if (M >= 256 && N >= 256 && tiles_big >= 128) return run_gemm_f16<Tile<256, 256, 128, 2, 4>, OUT_F16>(a, b, c, M, N, K, s);
+  // UNIT_AMD_GEMM_F16_VARIANT pins a tile shape per process (measurement aid)
+  switch (tuning_override("UNIT_AMD_GEMM_F16_VARIANT")) {
+    case 1: return run_gemm_f16<Tile<256, 256, 128, 2, 4>, OUT_F16>(a, b, c, M, N, K, s);
+    case 2: return run_gemm_f16<Tile<256, 256, 64, 2, 4>, OUT_F16>(a, b, c, M, N, K, s);
+    case 3: return run_gemm_f16<Tile<256, 256, 128, 2, 2>, OUT_F16>(a, b, c, M, N, K, s);
+    case 4: return run_gemm_f16<Tile<256, 256, 128, 4, 2>, OUT_F16>(a, b, c, M, N, K, s);
+    case 5: return run_gemm_f16<Tile<256, 256, 64, 4, 2>, OUT_F16, 2>(a, b, c, M, N, K, s);
+    case 6: return run_gemm_f16<Tile<128, 256, 128, 4, 2>, OUT_F16>(a, b, c, M, N, K, s);
+    default: break;
+  }
+  // 64 (m) x 128 (n) wave tiles: measured 8-10 % faster than 128 x 64 (512-byte row runs per wave in the write-back)
+  if (M >= 256 && N >= 256 && tiles_big >= 128) return run_gemm_f16<Tile<256, 256, 128, 4, 2>, OUT_F16>(a, b, c, M, N, K, s);
   return run_gemm_f16<Tile<128, 128, 64, 2, 2>, OUT_F16>(a, b, c, M, N, K, s);
 }
 

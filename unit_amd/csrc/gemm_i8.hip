@@ -116,6 +116,7 @@ int dense(const void *a, const void *w, void *c, int M, int N, int K, unit_strea
     case 12: if (!PACKED && K % 128 == 0) return run_dense_dma<Tile<256, 256, 128, 2, 4>, 2>(a, w, c, M, N, K, s); break;
     case 13: if (PACKED) return run_dense_mixed(a, w, c, M, N, K, s); break;
     case 14: return run_dense<Tile<256, 256, 128, 2, 4>, PACKED>(a, w, c, M, N, K, s);
+    case 15: return run_dense<Tile<256, 256, 128, 4, 2>, PACKED>(a, w, c, M, N, K, s);
     default: break;
   }
   if (M >= 256 && N >= 256 && tiles_big >= 128) return run_dense<Tile<256, 256, 128, 2, 4>, PACKED>(a, w, c, M, N, K, s);
