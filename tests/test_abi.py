@@ -36,6 +36,15 @@ def test_conv_desc_matches_the_header_struct():
     assert ctypes.sizeof(_lib.ConvDesc) == 4 * len(fields)
 
 
+def test_conv3d_desc_matches_the_header_struct():
+    from unit_amd import _lib
+    text = open(os.path.join(ROOT, "include", "unit_amd.h")).read()
+    body = re.search(r"typedef struct unit_conv3d_desc \{(.*?)\} unit_conv3d_desc;", text, flags=re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    fields = [f.strip() for decl in re.findall(r"int32_t ([^;]+);", body) for f in decl.split(",")]
+    assert fields == [f for f, _ in _lib.Conv3dDesc._fields_]
+
+
 def test_out_hw_and_error_paths_without_gpu():
     from unit_amd import _lib
     L = _lib.load()
@@ -60,6 +69,14 @@ def test_out_hw_and_error_paths_without_gpu():
     assert L.unit_conv2d_nchwc_u8s8s32(ctypes.byref(bad), 1, 1, 1, None) == -1
     pad = _lib.ConvDesc(1, 16, 8, 8, 16, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 16)  # fp16 op has no padding argument
     assert L.unit_conv2d_nchw16c_f16f32(ctypes.byref(pad), 1, 1, 1, None) == -1
+    # the fused signed form and the 3-D operator validate the same way
+    assert L.unit_conv2d_nchwc_s8s8s32_fused(ctypes.byref(bad), 1, 1, None, 11, 1, None) == -1
+    assert L.unit_conv2d_nchwc_s8s8s32_fused(None, 1, 1, None, 11, 1, None) == -1 and b"null" in L.unit_last_error()
+    d3 = _lib.Conv3dDesc(1, 24, 16, 8, 8, 16, 3, 3, 3, 1)  # C % 16 != 0
+    assert L.unit_conv3d_ncdhwc_s8s8s32(ctypes.byref(d3), 1, 1, 1, None) == -1 and b"multiples of 16" in L.unit_last_error()
+    d3 = _lib.Conv3dDesc(1, 16, 2, 8, 8, 16, 3, 3, 3, 1)   # kernel deeper than the input
+    assert L.unit_conv3d_ncdhwc_s8s8s32(ctypes.byref(d3), 1, 1, 1, None) == -1 and b"window" in L.unit_last_error()
+    assert L.unit_conv_variant_count() >= 70
     with pytest.raises(ValueError):
         _lib.check(-1)
 

@@ -18,6 +18,11 @@ def test_ops_refuse_cpu_tensors_instead_of_falling_back():
         U.gemm_fp16(torch.zeros((4, 8), dtype=torch.float16), torch.zeros((8, 4), dtype=torch.float16))
     with pytest.raises(TypeError):
         U.conv2d_NCHWc_int8(np.zeros((1, 4, 8, 8, 16), np.uint8), wt, 1, 1)
+    with pytest.raises(ValueError, match="GPU"):
+        U.conv2d_NCHWc_int8_fused(data.view(torch.int8), wt, None, 11, 1, 1)
+    with pytest.raises(ValueError, match="GPU"):
+        U.conv3d_NCDHWc_int8(torch.zeros((1, 1, 4, 8, 8, 16), dtype=torch.int8),
+                             torch.zeros((1, 1, 3, 3, 3, 4, 16, 4), dtype=torch.int8))
 
 
 def test_conv_out_hw_matches_reference_shapes():
