@@ -77,6 +77,10 @@ def test_out_hw_and_error_paths_without_gpu():
     d3 = _lib.Conv3dDesc(1, 16, 2, 8, 8, 16, 3, 3, 3, 1)   # kernel deeper than the input
     assert L.unit_conv3d_ncdhwc_s8s8s32(ctypes.byref(d3), 1, 1, 1, None) == -1 and b"window" in L.unit_last_error()
     assert L.unit_conv_variant_count() >= 70
+    # size limit: every tensor must stay below 2^31 bytes (32-bit offsets in the kernels)
+    huge = _lib.ConvDesc(4096, 256, 56, 56, 256, 1, 1, 1, 1, 0, 0, 0, 0, 1, 1, 16)
+    assert L.unit_conv2d_nchwc_u8s8s32(ctypes.byref(huge), 1, 1, 1, None) == -1 and b"2^31" in L.unit_last_error()
+    assert L.unit_dense_u8s8s32(1, 1, 1, 65536, 65536, 16, None) == -1 and b"2^31" in L.unit_last_error()
     with pytest.raises(ValueError):
         _lib.check(-1)
 

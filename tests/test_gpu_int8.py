@@ -68,6 +68,22 @@ def test_dense_packed_weights_direct_to_registers(dev, oracle, monkeypatch, M, N
     assert np.array_equal(out.cpu().numpy(), oracle.c_dense(a, wp)), U.last_variant()
 
 
+def test_dense_largest_output(dev, oracle):
+    """An output just below the 2^31-byte limit (23168^2 int32 = 2.147 GB): 32-bit offsets must not wrap."""
+    M = N = 23168
+    K = 32
+    assert M * N * 4 < 2 ** 31 <= (M + 128) * N * 4
+    a = rng.uniform_u8((M, K), 71)
+    w = rng.uniform_s8((N, K), 72)
+    out = U.dense(_t(a, dev), _t(w, dev))
+    torch.cuda.synchronize()
+    for rows in (slice(0, 64), slice(M // 2 - 32, M // 2 + 32), slice(M - 64, M)):
+        ref = a[rows].astype(np.int64) @ w.astype(np.int64).T
+        assert np.array_equal(out[rows].cpu().numpy().astype(np.int64), ref), U.last_variant()
+    del out
+    torch.cuda.empty_cache()
+
+
 def test_dense_extremes(dev, oracle):
     """255 x -128 everywhere: the largest negative accumulation (K * -32640), and 255 x 127."""
     M, N, K = 64, 128, 4096
