@@ -46,6 +46,10 @@ const char *unit_last_variant(void);
  * UNIT_AMD_CONV_VARIANT=1..count pins one per process, as the reference pins a schedule index
  * through the tensorizer.tune globals (python/tensorizer/tune.py:3-16). */
 int unit_conv_variant_count(void);
+/* 1 if variant 0..count-1 takes its operands straight from global memory into MFMA fragments
+ * (the kind the convolutions on prepared weights use), 0 if it stages them in LDS, -1 if there
+ * is no such variant.  For the tuner; no counterpart in the reference. */
+int unit_conv_variant_is_direct(int32_t variant);
 
 /* Geometry of one 2-D convolution; C and K are the channel counts as stored in the blocked
  * tensors (already rounded up: C % cb == 0, K % 16 == 0, apps/cpu/kernel/conv2d.py:18-22). */
@@ -168,6 +172,38 @@ int unit_prepack_dense_weight_s8(const void *src, void *dst, int32_t N, int32_t 
  * (python/tensorizer/ops/gpu.py:29-31).  O % 16 == 0, I % 16 == 0. */
 int unit_prepack_conv_weight_f16(const void *src, void *dst, int32_t O, int32_t I, int32_t KH,
                                  int32_t KW, unit_stream_t stream);
+
+/* ------------------------------------------------------------------ prepared weights */
+
+/* Convolution weights re-ordered once into the MFMA fragment order of the kernels, with the
+ * per-channel term of the u8 shift (128 * sum of the channel's weights) precomputed.  The
+ * reference's compiled graphs hold the same two pieces as constant sub-graphs next to the
+ * convolution: the weight layout chain (apps/cpu/relay/result.log:8-13) and sum(w) over
+ * (I, KH, KW) (result.log:15-16).  A convolution on prepared weights reads a lane's fragment with
+ * one 16-byte load and accumulates no weight sums in its reduction loop.
+ *
+ * weight: the blocked layout the convolutions above take, K and C multiples of 16:
+ *   elem_bytes 1: s8 (K/16, C/16, KH, KW, 4, 16, 4);  2: f16 (K/16, C/16, KH, KW, 16 in, 16 out).
+ * prepared: unit_conv2d_prepared_weight_bytes() bytes, 16-byte aligned, owned by the caller:
+ *   [ceil(K/32)][k-step][64 lanes][16 bytes] (+ int32 addend[ceil(K/32) * 32] for int8); it depends
+ *   on the weight only, not on the image size, stride or padding. */
+int unit_conv2d_prepared_weight_bytes(int32_t K, int32_t C, int32_t KH, int32_t KW, int32_t elem_bytes,
+                                      size_t *bytes);
+int unit_conv2d_prepare_weight(int32_t K, int32_t C, int32_t KH, int32_t KW, int32_t elem_bytes,
+                               const void *weight, void *prepared, unit_stream_t stream);
+
+/* The convolutions above on prepared weights; same results (int8: bit for bit; fp16: the same
+ * products summed in the same order).  16-channel blocks only (d->cb == 16); int8 windows of at
+ * most 31 positions.  Replace the same reference calls as unit_conv2d_nchwc_u8s8s32
+ * (apps/cpu/kernel/conv2d.py:50-51), unit_conv2d_nchwc_s8s8s32_fused (result.log:3-26) and
+ * unit_conv2d_nchw16c_f16f32 (python/tensorizer/ops/gpu.py:8-53). */
+int unit_conv2d_nchwc_u8s8s32_prepared(const unit_conv_desc *d, const void *data, const void *prepared,
+                                       void *out, unit_stream_t stream);
+int unit_conv2d_nchwc_s8s8s32_fused_prepared(const unit_conv_desc *d, const void *data, const void *prepared,
+                                             const int32_t *bias, int32_t scale, void *out,
+                                             unit_stream_t stream);
+int unit_conv2d_nchw16c_f16f32_prepared(const unit_conv_desc *d, const void *a, const void *prepared,
+                                        void *out, unit_stream_t stream);
 
 /* ------------------------------------------------------------------ diagnostics */
 

@@ -1,0 +1,199 @@
+"""Convolutions on prepared (MFMA-fragment-ordered) weights, through the C ABI: the prepared buffer
+against its index formula, and the results against the CPU oracle (int8: bit-exact; fp16: 1e-2
+max-rel against float64, and bit for bit against the convolution on the reference's layout)."""
+import numpy as np
+import pytest
+import torch
+
+import unit_amd as U
+from unit_amd import rng
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-2
+
+
+def _t(a, dev):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def _fragments_i8(wt):
+    """prepared[kb][s][lane][16] and addend[kb * 32 + c] from (K/16, C/16, KH, KW, 4, 16, 4) s8, by the index
+    formula: lane -> channel kb * 32 + lane % 32, tap 2 s + lane / 32, byte 4 e + i -> input channel 4 e + i."""
+    ko, cc, kh, kw = wt.shape[:4]
+    K, ntaps = ko * 16, cc * kh * kw
+    nsteps, kblocks = (ntaps + 1) // 2, (K + 31) // 32
+    # w[k][tap][ci16]
+    w = wt.reshape(ko, ntaps, 4, 16, 4).transpose(0, 3, 1, 2, 4).reshape(K, ntaps, 16)
+    full = np.zeros((kblocks * 32, nsteps * 2, 16), np.int8)
+    full[:K, :ntaps] = w
+    frag = full.reshape(kblocks, 32, nsteps, 2, 16).transpose(0, 2, 3, 1, 4).reshape(kblocks, nsteps, 64, 16)
+    addend = np.zeros(kblocks * 32, np.int32)
+    addend[:K] = 128 * w.astype(np.int64).sum(axis=(1, 2))
+    return frag, addend
+
+
+def _fragments_f16(b):
+    """prepared[kb][tap][lane][8 halves] from (K/16, C/16, KH, KW, 16 in, 16 out) f16: lane -> channel
+    kb * 32 + lane % 32, input channels 8 (lane / 32) .. + 8."""
+    ko, cc, kh, kw = b.shape[:4]
+    K, ntaps = ko * 16, cc * kh * kw
+    kblocks = (K + 31) // 32
+    w = b.reshape(ko, ntaps, 16, 16).transpose(0, 3, 1, 2).reshape(K, ntaps, 16)  # [k][tap][ci]
+    full = np.zeros((kblocks * 32, ntaps, 16), np.float16)
+    full[:K] = w
+    return full.reshape(kblocks, 32, ntaps, 2, 8).transpose(0, 2, 3, 1, 4).reshape(kblocks, ntaps, 64, 8)
+
+
+@pytest.mark.parametrize("K,C,ks", [(64, 64, 3), (48, 16, 3), (16, 32, 1), (96, 80, (1, 3))])
+def test_prepared_buffer_int8(dev, K, C, ks):
+    kh, kw = (ks, ks) if isinstance(ks, int) else ks
+    wt = rng.uniform_s8((K // 16, C // 16, kh, kw, 4, 16, 4), K + C)
+    p = U.prepare_conv2d_weight(_t(wt, dev))
+    torch.cuda.synchronize()
+    frag, addend = _fragments_i8(wt)
+    buf = p.buf.cpu().numpy()
+    assert buf.size == frag.size + addend.size * 4
+    assert np.array_equal(buf[:frag.size].view(np.int8).reshape(frag.shape), frag)
+    assert np.array_equal(buf[frag.size:].view(np.int32), addend)
+
+
+@pytest.mark.parametrize("K,C,ks", [(64, 64, 3), (48, 16, 1), (16, 48, 2)])
+def test_prepared_buffer_fp16(dev, K, C, ks):
+    b = rng.normal_f16((K // 16, C // 16, ks, ks, 16, 16), K + C)
+    p = U.prepare_conv2d_weight(_t(b, dev))
+    torch.cuda.synchronize()
+    frag = _fragments_f16(b)
+    buf = p.buf.cpu().numpy()
+    assert buf.size == frag.size * 2
+    assert np.array_equal(buf.view(np.float16).reshape(frag.shape), frag)
+
+
+CONV_CASES = [
+    # N, C, H, W, K, kernel, stride, pad, dilation
+    (1, 64, 56, 56, 64, 3, 1, 1, 1),       # BASELINE config (1)
+    (2, 32, 9, 7, 32, 3, 1, 1, 1),         # tiny, ragged pixel count
+    (1, 16, 8, 8, 48, 1, 2, 0, 1),         # one tap (half a k-step), K not a multiple of 32
+    (1, 16, 9, 9, 48, 3, 1, 0, 1),         # 9 taps, no padding: the kernel without tap masks on an odd tap count
+    (3, 64, 14, 14, 128, 1, 1, 0, 1),      # 1x1 = GEMM
+    (1, 256, 14, 14, 512, 3, 2, 1, 1),
+    (1, 512, 7, 7, 512, 3, 1, 1, 1),
+    (2, 16, 12, 12, 32, 3, 1, 2, 2),       # dilation 2
+    (1, 48, 10, 10, 80, 5, (2, 1), (2, 0), 1),   # anisotropic stride / pad, 5x5, 75 taps
+    (32, 64, 56, 56, 256, 1, 1, 0, 1),     # ResNet-50 batch 32 layers
+    (32, 256, 14, 14, 256, 3, 1, 1, 1),
+    (8, 512, 7, 7, 2048, 1, 1, 0, 1),
+]
+
+
+@pytest.mark.parametrize("N,C,H,W,K,ks,stride,pad,dil", CONV_CASES)
+def test_conv2d_prepared_bit_exact(dev, oracle, N, C, H, W, K, ks, stride, pad, dil):
+    data = rng.uniform_u8((N, C // 16, H, W, 16), 7 * C + H)
+    wt = rng.uniform_s8((K // 16, C // 16, ks, ks, 4, 16, 4), 3 * K + ks)
+    ref = oracle.c_conv2d_nchwc(data, wt, stride, pad, dil)
+    p = U.prepare_conv2d_weight(_t(wt, dev))
+    out = U.conv2d_NCHWc_int8(_t(data, dev), p, stride, pad, dil, "int32", "NCHW16c", "NCHW16c")
+    torch.cuda.synchronize()
+    assert "prep" in U.last_variant()
+    assert tuple(out.shape) == ref.shape
+    assert np.array_equal(out.cpu().numpy(), ref), U.last_variant()
+
+
+@pytest.mark.parametrize("N,C,H,W,K,ks,stride,pad", [
+    (2, 80, 9, 11, 96, 3, 1, 1),    # 45 taps: odd, zero padding, ragged tiles
+    (1, 32, 5, 5, 16, 1, 1, 0),     # one k-step: k-groups beyond the first have nothing to do
+    (3, 256, 7, 7, 160, 3, 2, 1),   # a long reduction over few pixels
+    (1, 48, 8, 8, 32, 3, 1, 0),     # 27 taps without padding
+])
+def test_conv2d_prepared_every_direct_variant(dev, oracle, monkeypatch, N, C, H, W, K, ks, stride, pad):
+    """u8 and fused signed form on every direct variant (ids of staged variants fall back to a direct one)."""
+    from unit_amd import _lib
+    data = rng.uniform_u8((N, C // 16, H, W, 16), 11 * C + H)
+    xs = (data ^ 0x80).view(np.int8)
+    wt = rng.uniform_s8((K // 16, C // 16, ks, ks, 4, 16, 4), 5 * K + ks)
+    bias = rng.uniform_s8((K,), 5).astype(np.int32) * 1001
+    ref = oracle.c_conv2d_nchwc(data, wt, stride, pad, 1)
+    ref_fused = oracle.conv2d_nchwc_int8_fused(xs, wt, bias, -7, stride, pad, 1, conv=oracle.c_conv2d_nchwc)
+    d, x, tb = _t(data, dev), _t(xs, dev), _t(bias, dev)
+    p = U.prepare_conv2d_weight(_t(wt, dev))
+    names = set()
+    for v in range(1, _lib.load().unit_conv_variant_count() + 1):
+        monkeypatch.setenv("UNIT_AMD_CONV_VARIANT", str(v))
+        out = U.conv2d_NCHWc_int8(d, p, stride, pad)
+        torch.cuda.synchronize()
+        names.add(U.last_variant())
+        assert np.array_equal(out.cpu().numpy(), ref), (v, U.last_variant())
+        out = U.conv2d_NCHWc_int8_fused(x, p, tb, -7, stride, pad)
+        torch.cuda.synchronize()
+        names.add(U.last_variant())
+        assert np.array_equal(out.cpu().numpy(), ref_fused), (v, U.last_variant())
+    assert len(names) >= 30 and all(n.startswith(("i8prep", "s8prep")) for n in names), names
+
+
+FP16_CASES = [
+    # N, C, H, W, K, kernel, stride
+    (1, 64, 16, 18, 64, 3, 1),
+    (1, 16, 9, 9, 16, 1, 1),
+    (2, 32, 12, 10, 48, 3, 2),
+    (1, 256, 30, 30, 256, 3, 2),
+    (4, 128, 30, 30, 128, 3, 1),
+    (32, 256, 16, 16, 256, 3, 1),
+]
+
+
+@pytest.mark.parametrize("N,C,H,W,K,ks,stride", FP16_CASES)
+def test_conv2d_fp16_prepared(dev, oracle, N, C, H, W, K, ks, stride):
+    a = rng.normal_f16((N, C // 16, H, W, 16), 5 + C)
+    b = rng.normal_f16((K // 16, C // 16, ks, ks, 16, 16), 9 + K, 1.0 / np.sqrt(C * ks * ks))
+    ta = _t(a, dev)
+    out = U.conv2d_NCHW16c_OHWI16o(ta, U.prepare_conv2d_weight(_t(b, dev)), stride, stride, "float32")
+    torch.cuda.synchronize()
+    assert U.last_variant().startswith("f16prep")
+    ref = oracle.conv2d_nchw16c_f16(a, b, stride, stride)
+    assert tuple(out.shape) == ref.shape
+    floor = 1e-3 * np.abs(ref).max()
+    err = float((np.abs(out.cpu().numpy().astype(np.float64) - ref) / np.maximum(np.abs(ref), floor)).max())
+    assert err <= REL_TOL, (err, U.last_variant())
+
+
+def test_conv2d_fp16_prepared_every_direct_variant(dev, oracle, monkeypatch):
+    """Integer-valued data: fp32 accumulation is exact in any order, so every variant must reproduce the float64
+    reference bit for bit; and on random data the prepared and the plain convolution of one variant agree bit
+    for bit (same products, same summation order)."""
+    from unit_amd import _lib
+    N, C, H, W, K, ks, stride = 2, 80, 9, 11, 96, 3, 1
+    a = (rng.uniform_u8((N, C // 16, H, W, 16), 3 + C) % 7).astype(np.float16) - 3
+    b = (rng.uniform_u8((K // 16, C // 16, ks, ks, 16, 16), 4 + K) % 5).astype(np.float16) - 2
+    ra = rng.normal_f16(a.shape, 1)
+    rb = rng.normal_f16(b.shape, 2, 0.05)
+    ref = oracle.conv2d_nchw16c_f16(a, b, stride, stride)
+    ta, tra, trb = _t(a, dev), _t(ra, dev), _t(rb, dev)
+    p, rp = U.prepare_conv2d_weight(_t(b, dev)), U.prepare_conv2d_weight(trb)
+    names = set()
+    for v in range(1, _lib.load().unit_conv_variant_count() + 1):
+        monkeypatch.setenv("UNIT_AMD_CONV_VARIANT", str(v))
+        try:
+            out = U.conv2d_NCHW16c_OHWI16o(ta, p, stride, stride)
+        except ValueError as e:  # a variant may only be refused for its LDS budget (parked fp32 partial tiles)
+            assert "LDS" in str(e), (v, str(e))
+            continue
+        torch.cuda.synchronize()
+        names.add(U.last_variant())
+        assert np.array_equal(out.cpu().numpy().astype(np.float64), ref), (v, U.last_variant())
+        plain = U.conv2d_NCHW16c_OHWI16o(tra, trb, stride, stride)
+        if U.last_variant().startswith("f16direct"):
+            prep = U.conv2d_NCHW16c_OHWI16o(tra, rp, stride, stride)
+            torch.cuda.synchronize()
+            assert torch.equal(plain, prep), (v, U.last_variant())
+    assert len(names) >= 15 and all(n.startswith("f16prep") for n in names), names
+
+
+def test_prepared_rejections(dev):
+    wt = _t(rng.uniform_s8((2, 2, 3, 3, 4, 16, 4), 1), dev)
+    p = U.prepare_conv2d_weight(wt)
+    with pytest.raises(ValueError):   # channel count of the data does not match
+        U.conv2d_NCHWc_int8(_t(rng.uniform_u8((1, 3, 8, 8, 16), 2), dev), p, 1, 1)
+    with pytest.raises(TypeError):    # int8 weights into the fp16 operator
+        U.conv2d_NCHW16c_OHWI16o(_t(rng.normal_f16((1, 2, 8, 8, 16), 3), dev), p, 1, 1)
+    with pytest.raises(ValueError):   # 4-channel blocks have no prepared form
+        U.prepare_conv2d_weight(_t(rng.uniform_s8((2, 1, 3, 3, 1, 16, 4), 1), dev))

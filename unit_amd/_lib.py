@@ -15,6 +15,7 @@ SYMBOLS = (
     "unit_last_error",
     "unit_last_variant",
     "unit_conv_variant_count",
+    "unit_conv_variant_is_direct",
     "unit_conv_out_hw",
     "unit_conv2d_nchwc_u8s8s32",
     "unit_conv2d_nchwc_s8s8s32_fused",
@@ -28,6 +29,11 @@ SYMBOLS = (
     "unit_prepack_conv_weight_s8",
     "unit_prepack_dense_weight_s8",
     "unit_prepack_conv_weight_f16",
+    "unit_conv2d_prepared_weight_bytes",
+    "unit_conv2d_prepare_weight",
+    "unit_conv2d_nchwc_u8s8s32_prepared",
+    "unit_conv2d_nchwc_s8s8s32_fused_prepared",
+    "unit_conv2d_nchw16c_f16f32_prepared",
     "unit_mfma_tile_i8",
     "unit_mfma_tile_f16",
     "unit_mfma_peak",
@@ -67,6 +73,7 @@ def load():
     L.unit_version.restype = ctypes.c_int
     L.unit_last_error.restype = ctypes.c_char_p
     L.unit_last_variant.restype = ctypes.c_char_p
+    L.unit_conv_variant_is_direct.argtypes = [i32]
     L.unit_conv_out_hw.argtypes = [dp, ctypes.POINTER(i32), ctypes.POINTER(i32)]
     L.unit_conv2d_nchwc_u8s8s32.argtypes = [dp, vp, vp, vp, vp]
     L.unit_conv2d_nchwc_s8s8s32_fused.argtypes = [dp, vp, vp, vp, i32, vp, vp]
@@ -80,6 +87,11 @@ def load():
     L.unit_prepack_conv_weight_s8.argtypes = [vp, vp, i32, i32, i32, i32, i32, vp]
     L.unit_prepack_dense_weight_s8.argtypes = [vp, vp, i32, i32, vp]
     L.unit_prepack_conv_weight_f16.argtypes = [vp, vp, i32, i32, i32, i32, vp]
+    L.unit_conv2d_prepared_weight_bytes.argtypes = [i32, i32, i32, i32, i32, ctypes.POINTER(ctypes.c_size_t)]
+    L.unit_conv2d_prepare_weight.argtypes = [i32, i32, i32, i32, i32, vp, vp, vp]
+    L.unit_conv2d_nchwc_u8s8s32_prepared.argtypes = [dp, vp, vp, vp, vp]
+    L.unit_conv2d_nchwc_s8s8s32_fused_prepared.argtypes = [dp, vp, vp, vp, i32, vp, vp]
+    L.unit_conv2d_nchw16c_f16f32_prepared.argtypes = [dp, vp, vp, vp, vp]
     L.unit_mfma_tile_i8.argtypes = [vp, vp, vp, vp]
     L.unit_mfma_tile_f16.argtypes = [vp, vp, vp, vp]
     L.unit_mfma_peak.argtypes = [i32, i32, i32, vp, vp]

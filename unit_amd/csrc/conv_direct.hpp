@@ -23,6 +23,13 @@
 // 128 * sum(w), accumulated on the side with v_dot4 (SHIFT).  Signed data needs neither; that is
 // the reference's fused form  (conv(x_s8 + 128, w) - 128 * sum(w) + bias) * scale
 // (apps/cpu/relay/result.log:3-26), which the epilogue's bias and scale complete.
+//
+// PREP: the weights come in the fragment order written by prepare_weight (conv_prepare.hip)
+// instead of the reference's layout: prepared[K/32][k-step][lane][16 bytes], so a lane's fragment of
+// a k-step is one 16-byte load (a wave reads 1 KiB of consecutive memory) instead of four dword
+// or eight 16-bit loads, and for u8 data the 128 * sum(w) correction is a per-channel constant
+// that prepare_weight left behind the fragments (passed here as the bias), so the reduction loop
+// does not accumulate weight sums.  The fragment that pads an odd tap count is zero.
 #pragma once
 #include "epilogues.hpp"
 #include "loaders.hpp"
@@ -95,7 +102,7 @@ __device__ __forceinline__ void store_block(const typename ConvEpilogue<Op>::Par
   }
 }
 
-template <class Op, class S, bool SHIFT>
+template <class Op, class S, bool SHIFT, bool PREP = false>
 __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ data, const char *__restrict__ wgt,
                                                      typename ConvEpilogue<Op>::Params ep, ConvGeom g, GridMap gm) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -149,6 +156,21 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
     int n = x0 + i * 32 + l32;
     n = n < ep.K ? n : ep.K - 1;
     xoff[i] = (u32)(n >> 4) * (u32)(g.ntaps * WTAP) + (kInt ? (u32)(n & 15) * 4u : (u32)(n & 15) * 2u + (u32)half * 256u);
+    if constexpr (PREP) {  // blocks past the last one re-read it
+      const int kb = min((x0 >> 5) + i, (ep.K - 1) >> 5);
+      xoff[i] = ((u32)(kb * nsteps) * 64u + (u32)lane) * 16u;
+    }
+  }
+  // per-channel addend read from memory (bias; with PREP and u8 data the shift correction): one
+  // wave contributes it, and the load is issued here so that its latency hides behind the loop
+  int addv[TX];
+#pragma unroll
+  for (int i = 0; i < TX; ++i) {
+    addv[i] = 0;
+    if constexpr (kInt) {
+      const int c = x0 + i * 32 + l32;
+      if (ep.bias != nullptr && wave == 0 && c < ep.K) addv[i] = ep.bias[c];
+    }
   }
   // data: byte offset of the window origin of this lane's pixel per 32-pixel block, and the set of
   // window positions (kh, kw) that fall inside the image (none for lanes past the last pixel)
@@ -202,6 +224,7 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
   auto fetch = [&](auto slot) __attribute__((always_inline)) {
     constexpr int U = decltype(slot)::value;
     const int t = kInt ? 2 * sf + half : sf;
+    const u32 xs = (u32)sf * 1024u;  // PREP: a k-step of a 32-channel block is 1 KiB
     const v2i e = ecur;
     sf = sf < slast ? sf + 1 : slast;
     ecur = tab[kInt ? 2 * sf + half : sf];
@@ -213,7 +236,9 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
 #pragma unroll
     for (int i = 0; i < TX; ++i) {
       const u32 o = xoff[i] + xk;
-      if constexpr (kInt) {
+      if constexpr (PREP) {
+        xf[U][i] = *reinterpret_cast<const v4i *>(wgt + xoff[i] + xs);
+      } else if constexpr (kInt) {
 #pragma unroll
         for (int d = 0; d < 4; ++d) xf[U][i][d] = *reinterpret_cast<const int *>(wgt + o + d * 64);
       } else {
@@ -247,7 +272,7 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
         if constexpr (SHIFT) v ^= (int)0x80808080;
         y[j][d] = v;
       }
-    if constexpr (SHIFT) {
+    if constexpr (SHIFT && !PREP) {
 #pragma unroll
       for (int i = 0; i < TX; ++i)
 #pragma unroll
@@ -311,22 +336,15 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
   }
 
   // the two 32-lane halves hold the weight sums of the two taps of every k-step
-  if constexpr (SHIFT) {
+  if constexpr (SHIFT && !PREP) {
 #pragma unroll
     for (int i = 0; i < TX; ++i) wsx[i] = (wsx[i] + __shfl_xor(wsx[i], 32)) << 7;
   }
   // what is added per channel before the scale: the shift correction and / or the bias; one wave
   // adds the bias.  `addend` is uniform over the workgroup.
   const bool addend = kInt && (SHIFT || ep.bias != nullptr);
-  if constexpr (kInt) {
-    if (ep.bias != nullptr && wave == 0) {
 #pragma unroll
-      for (int i = 0; i < TX; ++i) {
-        const int c = x0 + i * 32 + l32;
-        wsx[i] += c < ep.K ? ep.bias[c] : 0;
-      }
-    }
-  }
+  for (int i = 0; i < TX; ++i) wsx[i] += addv[i];
 
   if constexpr (KG == 1) {
     if (addend && half == 0) {

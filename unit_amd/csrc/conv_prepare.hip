@@ -1,0 +1,185 @@
+// One-time weight preparation for the direct convolution kernels, and the C-ABI entry points of
+// the convolutions that take prepared weights.  The reference's compiled graphs do the same kind
+// of work on the constant weight, outside the convolution: the transpose / reshape chain into the
+// blocked layout (apps/cpu/relay/result.log:8-13) and the per-channel weight sum of the u8 shift
+// (result.log:15-16); here both are folded into one buffer shaped for the MFMA fragments.
+#include "conv_plan.hpp"
+#include "conv_prepare.hpp"
+#include "mma_core.hpp"
+
+namespace unit {
+
+int conv_geom(const unit_conv_desc *d, int tapb, ConvGeom *g, const char *what);  // abi.hip
+const TunedConv *tuned_conv_i8_prepared(int *n);                                  // below
+int conv_u8_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
+                     const int *addend, void *out, hipStream_t s);  // conv_prepared_u8.hip
+int conv_s8_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
+                     const int *bias, int scale, void *out, hipStream_t s);  // conv_prepared_s8.hip
+int conv_f16_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *a, const void *w,
+                      void *out, hipStream_t s);  // conv_prepared_f16.hip
+
+namespace {
+
+// one workgroup (64 lanes) per (32-channel block, k-step): gathers the 1 KiB of fragments
+__global__ __launch_bounds__(64) void prepare_i8(const char *__restrict__ w, char *__restrict__ out, int K, int ntaps,
+                                                 int nsteps) {
+  const int blk = blockIdx.x, kb = blk / nsteps, s = blk - kb * nsteps;
+  const int lane = threadIdx.x, ko = kb * 32 + (lane & 31), t = 2 * s + (lane >> 5);
+  v4i v = {0, 0, 0, 0};
+  if (ko < K && t < ntaps) {
+    const char *src = w + ((size_t)(ko >> 4) * ntaps + t) * 256 + (ko & 15) * 4;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) v[d] = *reinterpret_cast<const int *>(src + d * 64);
+  }
+  *reinterpret_cast<v4i *>(out + ((size_t)blk * 64 + lane) * 16) = v;
+}
+
+// one wave per output channel: 128 * sum of its weights
+__global__ __launch_bounds__(64) void prepare_i8_addend(const char *__restrict__ w, int *__restrict__ addend, int K,
+                                                        int ntaps) {
+  const int ko = blockIdx.x, lane = threadIdx.x;
+  int sum = 0;
+  if (ko < K) {
+    const char *src = w + (size_t)(ko >> 4) * ntaps * 256 + (ko & 15) * 4;
+    for (int t = lane; t < ntaps; t += 64)
+#pragma unroll
+      for (int d = 0; d < 4; ++d)
+        sum = __builtin_amdgcn_sdot4(*reinterpret_cast<const int *>(src + (size_t)t * 256 + d * 64), 0x01010101, sum, false);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+  if (lane == 0) addend[ko] = sum << 7;
+}
+
+__global__ __launch_bounds__(64) void prepare_f16(const char *__restrict__ w, char *__restrict__ out, int K, int ntaps) {
+  const int blk = blockIdx.x, kb = blk / ntaps, s = blk - kb * ntaps;
+  const int lane = threadIdx.x, ko = kb * 32 + (lane & 31), half = lane >> 5;
+  v8h h;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) h[k] = (_Float16)0;
+  if (ko < K) {
+    const char *src = w + ((size_t)(ko >> 4) * ntaps + s) * 512 + (ko & 15) * 2 + half * 256;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) h[k] = *reinterpret_cast<const _Float16 *>(src + k * 32);
+  }
+  *reinterpret_cast<v8h *>(out + ((size_t)blk * 64 + lane) * 16) = h;
+}
+
+int check_weight_shape(const char *what, int K, int C, int KH, int KW, int elem_bytes, PreparedLayout *pl) {
+  if (elem_bytes != 1 && elem_bytes != 2) return fail(UNIT_E_ARG, "%s: elem_bytes must be 1 (int8) or 2 (fp16), got %d", what, elem_bytes);
+  if (K <= 0 || C <= 0 || KH <= 0 || KW <= 0) return fail(UNIT_E_ARG, "%s: K, C, KH, KW must be positive", what);
+  if (K % 16 || C % 16) return fail(UNIT_E_ARG, "%s: K and C must be multiples of 16 (got %d, %d)", what, K, C);
+  if (!fits((size_t)K * C * KH * KW * elem_bytes)) return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
+  *pl = prepared_layout(K, C, KH, KW, elem_bytes);
+  if (!fits(pl->total_bytes)) return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
+  return UNIT_OK;
+}
+
+// measured on MI355X by `python -m unit_amd.tune --prepared` (key: N*OH*OW, K, C, KH, KW, stride)
+const TunedConv kTunedI8Prepared[] = {
+#include "tuned_conv_i8_prepared.inc"
+    {0, 0, 0, 0, 0, 0, 0, 0, 0},
+};
+const TunedConv kTunedF16Prepared[] = {
+#include "tuned_conv_f16_prepared.inc"
+    {0, 0, 0, 0, 0, 0, 0, 0, 0},
+};
+
+// Prepared weights exist for the direct kernels only: a table entry or override that names a
+// staged variant falls back to the heuristic's direct choice.
+ConvPlan plan_prepared(const unit_conv_desc *d, const ConvGeom &g, int kbytes, const TunedConv *table, int ntable,
+                       bool int8) {
+  ConvPlan p = plan_conv(d, g.npix, kbytes, table, ntable, int8, true);
+  if (!kConvTiles[p.variant].direct) p = heuristic_plan(g.npix, d->K, kbytes, int8, true);
+  p.splits = 1;
+  return p;
+}
+
+int check_prepared_conv(const char *what, const unit_conv_desc *d, int tapb, ConvGeom *g) {
+  if (d->cb != 16) return fail(UNIT_E_ARG, "%s: prepared weights serve 16-channel blocks (got cb = %d)", what, d->cb);
+  if (int rc = conv_geom(d, tapb, g, what)) return rc;
+  if (tapb == 16 && d->KH * d->KW > 31) return fail(UNIT_E_ARG, "%s: window of %d x %d exceeds 31 positions", what, d->KH, d->KW);
+  if (!fits((size_t)g->npix * d->K * 4)) return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
+  return check_device();
+}
+
+}  // namespace
+}  // namespace unit
+
+extern "C" int unit_conv2d_prepared_weight_bytes(int32_t K, int32_t C, int32_t KH, int32_t KW, int32_t elem_bytes,
+                                                 size_t *bytes) {
+  using namespace unit;
+  const char *what = "unit_conv2d_prepared_weight_bytes";
+  if (!bytes) return fail(UNIT_E_ARG, "%s: null pointer", what);
+  PreparedLayout pl;
+  if (int rc = check_weight_shape(what, K, C, KH, KW, elem_bytes, &pl)) return rc;
+  *bytes = pl.total_bytes;
+  return UNIT_OK;
+}
+
+extern "C" int unit_conv2d_prepare_weight(int32_t K, int32_t C, int32_t KH, int32_t KW, int32_t elem_bytes,
+                                          const void *weight, void *prepared, unit_stream_t stream) {
+  using namespace unit;
+  const char *what = "unit_conv2d_prepare_weight";
+  if (!weight || !prepared) return fail(UNIT_E_ARG, "%s: null pointer", what);
+  PreparedLayout pl;
+  if (int rc = check_weight_shape(what, K, C, KH, KW, elem_bytes, &pl)) return rc;
+  if (int rc = check_device()) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int ntaps = (C / 16) * KH * KW;
+  const char *w = static_cast<const char *>(weight);
+  char *out = static_cast<char *>(prepared);
+  if (elem_bytes == 1) {
+    hipLaunchKernelGGL(prepare_i8, dim3(pl.kblocks * pl.nsteps), dim3(64), 0, s, w, out, K, ntaps, pl.nsteps);
+    hipLaunchKernelGGL(prepare_i8_addend, dim3(pl.kblocks * 32), dim3(64), 0, s, w,
+                       reinterpret_cast<int *>(out + pl.frag_bytes), K, ntaps);
+  } else {
+    hipLaunchKernelGGL(prepare_f16, dim3(pl.kblocks * pl.nsteps), dim3(64), 0, s, w, out, K, ntaps);
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "%s: launch: %s", what, hipGetErrorString(e));
+  set_variant("prepare_%s_k%d_s%d", elem_bytes == 1 ? "i8" : "f16", pl.kblocks, pl.nsteps);
+  return UNIT_OK;
+}
+
+extern "C" int unit_conv2d_nchwc_u8s8s32_prepared(const unit_conv_desc *d, const void *data, const void *prepared,
+                                                  void *out, unit_stream_t stream) {
+  using namespace unit;
+  const char *what = "unit_conv2d_nchwc_u8s8s32_prepared";
+  if (!d || !data || !prepared || !out) return fail(UNIT_E_ARG, "%s: null pointer", what);
+  ConvGeom g;
+  if (int rc = check_prepared_conv(what, d, 16, &g)) return rc;
+  const PreparedLayout pl = prepared_layout(d->K, d->C, d->KH, d->KW, 1);
+  const int ntable = (int)(sizeof(kTunedI8Prepared) / sizeof(kTunedI8Prepared[0])) - 1;
+  const ConvPlan p = plan_prepared(d, g, g.ntaps * 16, kTunedI8Prepared, ntable, true);
+  const char *w = static_cast<const char *>(prepared);
+  return conv_u8_prepared(p, d, g, data, w, reinterpret_cast<const int *>(w + pl.frag_bytes), out,
+                          static_cast<hipStream_t>(stream));
+}
+
+extern "C" int unit_conv2d_nchwc_s8s8s32_fused_prepared(const unit_conv_desc *d, const void *data,
+                                                        const void *prepared, const int32_t *bias, int32_t scale,
+                                                        void *out, unit_stream_t stream) {
+  using namespace unit;
+  const char *what = "unit_conv2d_nchwc_s8s8s32_fused_prepared";
+  if (!d || !data || !prepared || !out) return fail(UNIT_E_ARG, "%s: null pointer", what);
+  ConvGeom g;
+  if (int rc = check_prepared_conv(what, d, 16, &g)) return rc;
+  const int ntable = (int)(sizeof(kTunedI8Prepared) / sizeof(kTunedI8Prepared[0])) - 1;
+  const ConvPlan p = plan_prepared(d, g, g.ntaps * 16, kTunedI8Prepared, ntable, true);
+  return conv_s8_prepared(p, d, g, data, prepared, bias, scale, out, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int unit_conv2d_nchw16c_f16f32_prepared(const unit_conv_desc *d, const void *a, const void *prepared,
+                                                   void *out, unit_stream_t stream) {
+  using namespace unit;
+  const char *what = "unit_conv2d_nchw16c_f16f32_prepared";
+  if (!d || !a || !prepared || !out) return fail(UNIT_E_ARG, "%s: null pointer", what);
+  if (d->pt || d->pl || d->pb || d->pr) return fail(UNIT_E_ARG, "%s: the operator has no padding argument; pre-pad the data", what);
+  if (d->dh != 1 || d->dw != 1) return fail(UNIT_E_ARG, "%s: dilation must be 1", what);
+  ConvGeom g;
+  if (int rc = check_prepared_conv(what, d, 32, &g)) return rc;
+  const int ntable = (int)(sizeof(kTunedF16Prepared) / sizeof(kTunedF16Prepared[0])) - 1;
+  const ConvPlan p = plan_prepared(d, g, g.ntaps * 32, kTunedF16Prepared, ntable, false);
+  return conv_f16_prepared(p, d, g, a, prepared, out, static_cast<hipStream_t>(stream));
+}

@@ -1,0 +1,27 @@
+// Direct variants of the fused signed NCHW16c convolution, (conv(s8, s8) + bias) * scale, on
+// prepared weights.
+#include "conv_direct_host.hpp"
+
+namespace unit {
+
+int conv_s8_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
+                     const int *bias, int scale, void *out, hipStream_t s) {
+  const char *what = "unit_conv2d_nchwc_s8s8s32_fused_prepared";
+  const bool masked = d->pt || d->pl || d->pb || d->pr;
+#define UNIT_CONV_VARIANT(ID, BX, BY, BKB, WX, WY, PF, FF, KG)
+#define UNIT_CONV_DIRECT(ID, TX, TY, KG, D)                                                                             \
+  case ID:                                                                                                              \
+    return masked ? run_direct<OpI8, DirectShape<TX, TY, KG, D, true>, false, true>(what, "s8prep_c16", d, g, data, w,  \
+                                                                                     bias, scale, out, plan, s)         \
+                  : run_direct<OpI8, DirectShape<TX, TY, KG, D, false>, false, true>(what, "s8prep_c16", d, g, data, w, \
+                                                                                      bias, scale, out, plan, s);
+  switch (plan.variant) {
+#include "conv_variants.def"
+    default:
+      return fail(UNIT_E_ARG, "%s: unknown kernel variant %d", what, plan.variant);
+  }
+#undef UNIT_CONV_DIRECT
+#undef UNIT_CONV_VARIANT
+}
+
+}  // namespace unit

@@ -21,6 +21,7 @@ __all__ = [
     "conv2d_NCHWc_int8", "dense_dotprod", "dense", "conv2d_NCHW16c_OHWI16o", "gemm_fp16",
     "pack_nchwc", "unpack_nchwc", "prepack_conv_weight", "prepack_dense_weight",
     "prepack_conv_weight_f16", "conv_out_hw", "last_variant",
+    "PreparedConvWeight", "prepare_conv2d_weight",
 ]
 
 
@@ -87,6 +88,60 @@ def last_variant():
     return _lib.last_variant()
 
 
+# ------------------------------------------------------------------------------- prepared weights
+class PreparedConvWeight:
+    """Convolution weights in the MFMA fragment order of the kernels (see prepare_conv2d_weight).
+    Accepted wherever conv2d_NCHWc_int8, conv2d_NCHWc_int8_fused and conv2d_NCHW16c_OHWI16o take
+    a kernel."""
+
+    def __init__(self, buf, K, C, KH, KW, dtype):
+        self.buf, self.K, self.C, self.KH, self.KW, self.dtype = buf, K, C, KH, KW, dtype
+
+    def __repr__(self):
+        return f"PreparedConvWeight(K={self.K}, C={self.C}, KH={self.KH}, KW={self.KW}, dtype={self.dtype})"
+
+
+def prepare_conv2d_weight(kernel):
+    """Re-order a blocked convolution weight once for the direct kernels: the counterpart of the
+    constant sub-graphs the reference's compiled models keep next to each convolution (weight
+    layout chain apps/cpu/relay/result.log:8-13, sum(w) result.log:15-16).
+
+    kernel int8 (K/16, C/16, KH, KW, 4, 16, 4) or fp16 (K/16, C/16, KH, KW, 16 in, 16 out)
+    returns a PreparedConvWeight; convolutions on it give the same results as on `kernel`.
+    """
+    import ctypes
+    if isinstance(kernel, torch.Tensor) and kernel.dtype == torch.float16:
+        kernel = _dev(kernel, "kernel", torch.float16, 6)
+        ko, cc, kh, kw, ic, ob = kernel.shape
+        if (ic, ob) != (16, 16):
+            raise ValueError(f"kernel: expected (K/16, C/16, KH, KW, 16, 16), got {tuple(kernel.shape)}")
+        eb = 2
+    else:
+        kernel = _dev(kernel, "kernel", torch.int8, 7)
+        ko, cc, kh, kw, e, kb, i4 = kernel.shape
+        if (e, kb, i4) != (4, 16, 4):
+            raise ValueError(f"kernel: expected (K/16, C/16, KH, KW, 4, 16, 4), got {tuple(kernel.shape)}")
+        eb = 1
+    L = _lib.load()
+    nbytes = ctypes.c_size_t()
+    check(L.unit_conv2d_prepared_weight_bytes(ko * 16, cc * 16, kh, kw, eb, ctypes.byref(nbytes)))
+    buf = torch.empty(nbytes.value, dtype=torch.uint8, device=kernel.device)
+    check(L.unit_conv2d_prepare_weight(ko * 16, cc * 16, kh, kw, eb, kernel.data_ptr(), buf.data_ptr(), _stream()))
+    return PreparedConvWeight(buf, ko * 16, cc * 16, kh, kw, kernel.dtype)
+
+
+def _prepared_dims(kernel, data, want_dtype):
+    """(K/16, C/16, KH, KW) of a PreparedConvWeight after checking it against the data tensor."""
+    n, cc, h, w, cb = data.shape
+    if kernel.dtype != want_dtype:
+        raise TypeError(f"kernel: prepared from {kernel.dtype}, this operator takes {want_dtype}")
+    if cb != 16 or kernel.C != cc * 16:
+        raise ValueError(f"kernel: {kernel!r} does not match data {tuple(data.shape)} (16-channel blocks only)")
+    if kernel.buf.device != data.device:
+        raise ValueError("kernel: prepared on another device")
+    return kernel.K // 16, cc, kernel.KH, kernel.KW
+
+
 # ------------------------------------------------------------------------------- int8
 def conv2d_NCHWc_int8(data, kernel, stride, padding, dilation=1, out_dtype="int32", layout="NCHW16c",
                       out_layout="NCHW16c"):
@@ -101,19 +156,24 @@ def conv2d_NCHWc_int8(data, kernel, stride, padding, dilation=1, out_dtype="int3
     """
     import ctypes
     data = _dev(data, "data", torch.uint8, 5)
-    kernel = _dev(kernel, "kernel", torch.int8, 7)
+    prepared = isinstance(kernel, PreparedConvWeight)
+    if not prepared:
+        kernel = _dev(kernel, "kernel", torch.int8, 7)
     if out_dtype != "int32":
         raise ValueError(f"out_dtype: only 'int32' is supported, got {out_dtype!r}")
     _layout_block(layout, "layout")
     if _layout_block(out_layout, "out_layout") != 16:
         raise ValueError("out_layout: the output channel block is 16 (NCHW16c)")
     n, cc, h, w, cb = data.shape
-    ko, cc2, kh, kw, e, kb, i4 = kernel.shape
     if cb not in (4, 16):
         raise ValueError(f"data: channel block must be 16 or 4, got {cb}")
-    if (cc2, e, kb, i4) != (cc, cb // 4, 16, 4):
-        raise ValueError(f"kernel: shape {tuple(kernel.shape)} does not match data {tuple(data.shape)}; "
-                         f"expected (K/16, {cc}, KH, KW, {cb // 4}, 16, 4)")
+    if prepared:
+        ko, cc2, kh, kw = _prepared_dims(kernel, data, torch.int8)
+    else:
+        ko, cc2, kh, kw, e, kb, i4 = kernel.shape
+        if (cc2, e, kb, i4) != (cc, cb // 4, 16, 4):
+            raise ValueError(f"kernel: shape {tuple(kernel.shape)} does not match data {tuple(data.shape)}; "
+                             f"expected (K/16, {cc}, KH, KW, {cb // 4}, 16, 4)")
     sh, sw = _pair(stride, "stride")
     dh, dw = _pair(dilation, "dilation")
     pt, pl, pb, pr = _pad4(padding)
@@ -122,8 +182,12 @@ def conv2d_NCHWc_int8(data, kernel, stride, padding, dilation=1, out_dtype="int3
     oh, ow = ctypes.c_int32(), ctypes.c_int32()
     check(L.unit_conv_out_hw(ctypes.byref(d), ctypes.byref(oh), ctypes.byref(ow)))
     out = torch.empty((n, ko, oh.value, ow.value, 16), dtype=torch.int32, device=data.device)
-    check(L.unit_conv2d_nchwc_u8s8s32(ctypes.byref(d), data.data_ptr(), kernel.data_ptr(), out.data_ptr(),
-                                      _stream()))
+    if prepared:
+        check(L.unit_conv2d_nchwc_u8s8s32_prepared(ctypes.byref(d), data.data_ptr(), kernel.buf.data_ptr(),
+                                                   out.data_ptr(), _stream()))
+    else:
+        check(L.unit_conv2d_nchwc_u8s8s32(ctypes.byref(d), data.data_ptr(), kernel.data_ptr(), out.data_ptr(),
+                                          _stream()))
     return out
 
 
@@ -144,19 +208,24 @@ def conv2d_NCHWc_int8_fused(data, kernel, bias, scale, stride, padding, dilation
     """
     import ctypes
     data = _dev(data, "data", torch.int8, 5)
-    kernel = _dev(kernel, "kernel", torch.int8, 7)
+    prepared = isinstance(kernel, PreparedConvWeight)
+    if not prepared:
+        kernel = _dev(kernel, "kernel", torch.int8, 7)
     if out_dtype != "int32":
         raise ValueError(f"out_dtype: only 'int32' is supported, got {out_dtype!r}")
     _layout_block(layout, "layout")
     if _layout_block(out_layout, "out_layout") != 16:
         raise ValueError("out_layout: the output channel block is 16 (NCHW16c)")
     n, cc, h, w, cb = data.shape
-    ko, cc2, kh, kw, e, kb, i4 = kernel.shape
     if cb not in (4, 16):
         raise ValueError(f"data: channel block must be 16 or 4, got {cb}")
-    if (cc2, e, kb, i4) != (cc, cb // 4, 16, 4):
-        raise ValueError(f"kernel: shape {tuple(kernel.shape)} does not match data {tuple(data.shape)}; "
-                         f"expected (K/16, {cc}, KH, KW, {cb // 4}, 16, 4)")
+    if prepared:
+        ko, cc2, kh, kw = _prepared_dims(kernel, data, torch.int8)
+    else:
+        ko, cc2, kh, kw, e, kb, i4 = kernel.shape
+        if (cc2, e, kb, i4) != (cc, cb // 4, 16, 4):
+            raise ValueError(f"kernel: shape {tuple(kernel.shape)} does not match data {tuple(data.shape)}; "
+                             f"expected (K/16, {cc}, KH, KW, {cb // 4}, 16, 4)")
     if bias is not None:
         if bias.dtype != torch.int32 or bias.numel() != ko * 16 or bias.device != data.device:
             raise ValueError(f"bias: expected {ko * 16} int32 values on {data.device}")
@@ -172,9 +241,9 @@ def conv2d_NCHWc_int8_fused(data, kernel, bias, scale, stride, padding, dilation
     oh, ow = ctypes.c_int32(), ctypes.c_int32()
     check(L.unit_conv_out_hw(ctypes.byref(d), ctypes.byref(oh), ctypes.byref(ow)))
     out = torch.empty((n, ko, oh.value, ow.value, 16), dtype=torch.int32, device=data.device)
-    check(L.unit_conv2d_nchwc_s8s8s32_fused(ctypes.byref(d), data.data_ptr(), kernel.data_ptr(),
-                                            bias.data_ptr() if bias is not None else None, scale, out.data_ptr(),
-                                            _stream()))
+    fn = L.unit_conv2d_nchwc_s8s8s32_fused_prepared if prepared else L.unit_conv2d_nchwc_s8s8s32_fused
+    check(fn(ctypes.byref(d), data.data_ptr(), kernel.buf.data_ptr() if prepared else kernel.data_ptr(),
+             bias.data_ptr() if bias is not None else None, scale, out.data_ptr(), _stream()))
     return out
 
 
@@ -267,6 +336,19 @@ def conv2d_NCHW16c_OHWI16o(a, b, stride_h, stride_w, out_type="float32"):
     if out_type != "float32":
         raise ValueError(f"out_type: only 'float32' is supported, got {out_type!r}")
     a = _dev(a, "a", torch.float16, (4, 5))
+    if isinstance(b, PreparedConvWeight):
+        if a.dim() != 5:
+            raise ValueError("a: prepared weights take the blocked (N, C/16, H, W, 16) operand")
+        ko, cc, kh, kw = _prepared_dims(b, a, torch.float16)
+        n, _, h, w, _ = a.shape
+        d = ConvDesc(n, cc * 16, h, w, ko * 16, kh, kw, int(stride_h), int(stride_w), 0, 0, 0, 0, 1, 1, 16)
+        L = _lib.load()
+        oh, ow = ctypes.c_int32(), ctypes.c_int32()
+        check(L.unit_conv_out_hw(ctypes.byref(d), ctypes.byref(oh), ctypes.byref(ow)))
+        out = torch.empty((n, ko, oh.value, ow.value, 16), dtype=torch.float32, device=a.device)
+        check(L.unit_conv2d_nchw16c_f16f32_prepared(ctypes.byref(d), a.data_ptr(), b.buf.data_ptr(), out.data_ptr(),
+                                                    _stream()))
+        return out
     b = _dev(b, "b", torch.float16, (4, 6))
     if a.dim() == 4 and b.dim() == 4:
         if a.shape[1] % 16 or b.shape[0] % 16 or b.shape[1] != a.shape[1]:

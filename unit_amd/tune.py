@@ -6,9 +6,11 @@ keyed by (ashape, bshape, strides)).
 Here the candidates are the tile variants compiled into libunit_amd.so.  For every layer shape
 each variant is run through the C ABI, checked bit for bit against the library's default choice,
 and timed with HIP events; the fastest goes into unit_amd/csrc/tuned_conv_{i8,f16}.inc, which the
-library's planner consults first (rebuild after tuning).  Needs an MI355X.
+library's planner consults first (rebuild after tuning).  Needs an MI355X.  With --prepared the
+convolutions on prepared weights are tuned (direct variants only, 16-channel blocks only) into
+tuned_conv_{i8,f16}_prepared.inc.
 
-    python -m unit_amd.tune [--dtype i8|f16] [--nets resnet50:32,resnet18:1] [--iters 20] [--write]
+    python -m unit_amd.tune [--dtype i8|f16] [--prepared] [--nets resnet50:32,resnet18:1] [--iters 20] [--write]
 """
 import argparse
 import ctypes
@@ -28,7 +30,7 @@ def _shapes(spec):
     return out
 
 
-def tune(spec, iters=20, verbose=True, dtype="i8"):
+def tune(spec, iters=20, verbose=True, dtype="i8", prepared=False):
     import torch
 
     from . import _lib, last_variant
@@ -64,6 +66,8 @@ def tune(spec, iters=20, verbose=True, dtype="i8"):
             cb = WL.channel_block(s.C) if dtype == "i8" else 16
             if s.C % cb and dtype != "i8":
                 continue  # the fp16 operator needs C % 16 == 0
+            if prepared and (cb != 16 or (dtype == "i8" and s.KH * s.KW > 31)):
+                continue  # no prepared form
             cp = -(-s.C // cb) * cb
             oh, ow = WL.out_hw(s)
             key = (batch * oh * ow, s.K, cp, s.KH, s.KW, s.stride)
@@ -85,6 +89,10 @@ def tune(spec, iters=20, verbose=True, dtype="i8"):
                 out = torch.empty((batch, s.K // 16, oh, ow, 16), dtype=torch.float32, device=dev)
                 desc = _lib.ConvDesc(batch, cp, hp, wp, s.K, s.KH, s.KW, s.stride, s.stride, 0, 0, 0, 0, 1, 1, 16)
                 entry = L.unit_conv2d_nchw16c_f16f32
+            if prepared:
+                from .ops import prepare_conv2d_weight
+                wt = prepare_conv2d_weight(wt).buf
+                entry = L.unit_conv2d_nchwc_u8s8s32_prepared if dtype == "i8" else L.unit_conv2d_nchw16c_f16f32_prepared
 
             def call():
                 return entry(ctypes.byref(desc), data.data_ptr(), wt.data_ptr(), out.data_ptr(), stream)
@@ -99,9 +107,11 @@ def tune(spec, iters=20, verbose=True, dtype="i8"):
             default_us = best[0]
             timings = {}  # kernel name -> us, every candidate (kept in the --json dump)
             combos = [(1, 0), (1, 1), (1, 2), (1, 4)]  # (k-splits, channel tiles per panel)
-            if dtype == "i8":
+            if dtype == "i8" and not prepared:
                 combos += [(n, 0) for n in (2, 4, 8, 16, 32)]
             for v in range(num_variants):
+                if prepared and L.unit_conv_variant_is_direct(v) != 1:
+                    continue
                 for splits, panel in combos:
                     if splits > 1 and (splits // 2) * key[0] * s.K > 256 * 256 * 256:
                         break  # the grid already covers the chip: more k-splits only add atomics
@@ -156,16 +166,17 @@ def main():
     ap.add_argument("--nets", default="resnet50:32,resnet18:1,single:1")
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--dtype", default="i8", choices=["i8", "f16"])
-    ap.add_argument("--write", action="store_true", help="rewrite csrc/tuned_conv_i8.inc")
+    ap.add_argument("--prepared", action="store_true", help="tune the convolutions on prepared weights")
+    ap.add_argument("--write", action="store_true", help="rewrite csrc/tuned_conv_<dtype>[_prepared].inc")
     ap.add_argument("--table", default=None, help="write the table here instead of csrc/tuned_conv_i8.inc")
     ap.add_argument("--json", default=None, help="also dump the raw results here")
     args = ap.parse_args()
-    results = tune(args.nets, args.iters, dtype=args.dtype)
+    results = tune(args.nets, args.iters, dtype=args.dtype, prepared=args.prepared)
     if args.json:
         json.dump(results, open(args.json, "w"), indent=1)
     if args.write or args.table:
         path = args.table or os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc",
-                                          f"tuned_conv_{args.dtype}.inc")
+                                          f"tuned_conv_{args.dtype}{'_prepared' if args.prepared else ''}.inc")
         n = write_table(results, path)
         print(f"wrote {n} entries to {path}; rebuild with `make -C {os.path.dirname(path)}`")
 
