@@ -124,7 +124,7 @@ def main():
             L.unit_conv2d_nchwc_u8s8s32(ctypes.byref(d), x.data_ptr(), w.data_ptr(), o.data_ptr(),
                                         torch.cuda.current_stream().cuda_stream)))
         call, prep = call_ref, None
-        if cb == 16 and args.weights == "prepared":
+        if args.weights == "prepared" and (cb == 16 or s.KW <= 8):
             # the constant weight is re-ordered once, before the timed region, as the reference's compiled
             # graphs fold the weight layout chain and sum(w) (apps/cpu/relay/result.log:8-16)
             prep = U.prepare_conv2d_weight(wt)
@@ -281,7 +281,7 @@ def main():
             o = torch.empty((batch, s.K // 16, oh, ow, 16), dtype=torch.int32, device=dev)
             desc = _lib.ConvDesc(batch, cp, s.H, s.W, s.K, s.KH, s.KW, s.stride, s.stride, s.pad, s.pad, s.pad, s.pad,
                                  1, 1, cb)
-            prep = prepared and cb == 16 and s.KH * s.KW <= 31
+            prep = prepared and (s.KH * s.KW <= 31 if cb == 16 else s.KW <= 8)
             if prep:
                 w = U.prepare_conv2d_weight(w).buf
             if fused:  # signed activations, bias and scale: the form the reference's quantized graphs run
@@ -450,10 +450,10 @@ def main():
         "config": {"workload": "ResNet-50 v1 conv stack (53 convolutions, 20 unique shapes), batch 32, int8 "
                                "u8 x s8 -> i32, NCHW16c / NCHW4c stem (BASELINE configs[4])",
                    "batch": BATCH, "ops_per_step": step_ops,
-                   "weights": ("NCHW16c layers: prepared once before the timed region (unit_conv2d_prepare_weight: "
-                               "MFMA fragment order + 128 * sum(w)), as the reference folds its weight layout chain "
-                               "and sum(w) into constants; NCHW4c stem: the reference's layout"
-                               if args.weights == "prepared" else "the reference's blocked layout in every call")},
+                   "weights": ("prepared once before the timed region (unit_conv2d_prepare_weight: MFMA fragment "
+                               "order + 128 * sum(w)), as the reference folds its weight layout chain and sum(w) "
+                               "into constants" if args.weights == "prepared"
+                               else "the reference's blocked layout in every call")},
         "pct_int8_mfma_peak": round(100 * value / PEAK_INT8_TOPS, 2),
         "host_wall_ms_per_step": round(wall_ms, 4),
         "launch": launch_mode,

@@ -182,19 +182,20 @@ int unit_prepack_conv_weight_f16(const void *src, void *dst, int32_t O, int32_t 
  * (I, KH, KW) (result.log:15-16).  A convolution on prepared weights reads a lane's fragment with
  * one 16-byte load and accumulates no weight sums in its reduction loop.
  *
- * weight: the blocked layout the convolutions above take, K and C multiples of 16:
- *   elem_bytes 1: s8 (K/16, C/16, KH, KW, 4, 16, 4);  2: f16 (K/16, C/16, KH, KW, 16 in, 16 out).
+ * weight: the blocked layout the convolutions above take, K a multiple of 16 and C of cb:
+ *   elem_bytes 1: s8 (K/16, C/cb, KH, KW, cb/4, 16, 4), cb = 16, or cb = 4 with KW <= 8 (the stem);
+ *   elem_bytes 2: f16 (K/16, C/16, KH, KW, 16 in, 16 out), cb = 16.
  * prepared: unit_conv2d_prepared_weight_bytes() bytes, 16-byte aligned, owned by the caller:
  *   [ceil(K/32)][k-step][64 lanes][16 bytes] (+ int32 addend[ceil(K/32) * 32] for int8); it depends
  *   on the weight only, not on the image size, stride or padding. */
-int unit_conv2d_prepared_weight_bytes(int32_t K, int32_t C, int32_t KH, int32_t KW, int32_t elem_bytes,
-                                      size_t *bytes);
-int unit_conv2d_prepare_weight(int32_t K, int32_t C, int32_t KH, int32_t KW, int32_t elem_bytes,
+int unit_conv2d_prepared_weight_bytes(int32_t K, int32_t C, int32_t KH, int32_t KW, int32_t cb,
+                                      int32_t elem_bytes, size_t *bytes);
+int unit_conv2d_prepare_weight(int32_t K, int32_t C, int32_t KH, int32_t KW, int32_t cb, int32_t elem_bytes,
                                const void *weight, void *prepared, unit_stream_t stream);
 
 /* The convolutions above on prepared weights; same results (int8: bit for bit; fp16: the same
- * products summed in the same order).  16-channel blocks only (d->cb == 16); int8 windows of at
- * most 31 positions.  Replace the same reference calls as unit_conv2d_nchwc_u8s8s32
+ * products summed in the same order).  d->cb == 16 with int8 windows of at most 31 positions, or
+ * (int8 only) d->cb == 4 with KW <= 8, KH <= 31 and no dilation along W.  Replace the same reference calls as unit_conv2d_nchwc_u8s8s32
  * (apps/cpu/kernel/conv2d.py:50-51), unit_conv2d_nchwc_s8s8s32_fused (result.log:3-26) and
  * unit_conv2d_nchw16c_f16f32 (python/tensorizer/ops/gpu.py:8-53). */
 int unit_conv2d_nchwc_u8s8s32_prepared(const unit_conv_desc *d, const void *data, const void *prepared,

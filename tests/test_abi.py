@@ -82,14 +82,20 @@ def test_out_hw_and_error_paths_without_gpu():
     assert L.unit_conv_variant_is_direct(-1) == -1 and L.unit_conv_variant_is_direct(len(kinds)) == -1
     # prepared weights: size formula ceil(K/32) * k-steps * 1 KiB (+ 128 bytes of addends per block for int8)
     nb = ctypes.c_size_t()
-    assert L.unit_conv2d_prepared_weight_bytes(256, 256, 3, 3, 1, ctypes.byref(nb)) == 0 and nb.value == 8 * 72 * 1024 + 8 * 128
-    assert L.unit_conv2d_prepared_weight_bytes(48, 16, 3, 3, 1, ctypes.byref(nb)) == 0 and nb.value == 2 * 5 * 1024 + 2 * 128
-    assert L.unit_conv2d_prepared_weight_bytes(48, 16, 3, 3, 2, ctypes.byref(nb)) == 0 and nb.value == 2 * 9 * 1024
-    assert L.unit_conv2d_prepared_weight_bytes(40, 16, 3, 3, 1, ctypes.byref(nb)) == -1 and b"multiples of 16" in L.unit_last_error()
-    assert L.unit_conv2d_prepared_weight_bytes(48, 16, 3, 3, 4, ctypes.byref(nb)) == -1 and b"elem_bytes" in L.unit_last_error()
-    assert L.unit_conv2d_prepare_weight(48, 16, 3, 3, 1, None, 1, None) == -1 and b"null" in L.unit_last_error()
-    c4 = _lib.ConvDesc(1, 4, 8, 8, 16, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 4)
-    assert L.unit_conv2d_nchwc_u8s8s32_prepared(ctypes.byref(c4), 1, 1, 1, None) == -1 and b"16-channel" in L.unit_last_error()
+    assert L.unit_conv2d_prepared_weight_bytes(256, 256, 3, 3, 16, 1, ctypes.byref(nb)) == 0 and nb.value == 8 * 72 * 1024 + 8 * 128
+    assert L.unit_conv2d_prepared_weight_bytes(48, 16, 3, 3, 16, 1, ctypes.byref(nb)) == 0 and nb.value == 2 * 5 * 1024 + 2 * 128
+    assert L.unit_conv2d_prepared_weight_bytes(48, 16, 3, 3, 16, 2, ctypes.byref(nb)) == 0 and nb.value == 2 * 9 * 1024
+    # 4-channel blocks: one k-step per (channel block, kh)
+    assert L.unit_conv2d_prepared_weight_bytes(64, 4, 7, 7, 4, 1, ctypes.byref(nb)) == 0 and nb.value == 2 * 7 * 1024 + 2 * 128
+    assert L.unit_conv2d_prepared_weight_bytes(64, 4, 9, 9, 4, 1, ctypes.byref(nb)) == -1 and b"KW <= 8" in L.unit_last_error()
+    assert L.unit_conv2d_prepared_weight_bytes(64, 4, 3, 3, 4, 2, ctypes.byref(nb)) == -1 and b"cb must be" in L.unit_last_error()
+    assert L.unit_conv2d_prepared_weight_bytes(40, 16, 3, 3, 16, 1, ctypes.byref(nb)) == -1 and b"multiple of 16" in L.unit_last_error()
+    assert L.unit_conv2d_prepared_weight_bytes(48, 16, 3, 3, 16, 4, ctypes.byref(nb)) == -1 and b"elem_bytes" in L.unit_last_error()
+    assert L.unit_conv2d_prepare_weight(48, 16, 3, 3, 16, 1, None, 1, None) == -1 and b"null" in L.unit_last_error()
+    c4 = _lib.ConvDesc(1, 4, 8, 8, 16, 3, 3, 1, 1, 1, 1, 1, 1, 1, 2, 4)
+    assert L.unit_conv2d_nchwc_u8s8s32_prepared(ctypes.byref(c4), 1, 1, 1, None) == -1 and b"dilation along W" in L.unit_last_error()
+    c8 = _lib.ConvDesc(1, 8, 8, 8, 16, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 8)
+    assert L.unit_conv2d_nchwc_u8s8s32_prepared(ctypes.byref(c8), 1, 1, 1, None) == -1 and b"cb must be" in L.unit_last_error()
     big = _lib.ConvDesc(1, 16, 20, 20, 16, 7, 7, 1, 1, 0, 0, 0, 0, 1, 1, 16)
     assert L.unit_conv2d_nchwc_s8s8s32_fused_prepared(ctypes.byref(big), 1, 1, None, 1, 1, None) == -1 and b"31 positions" in L.unit_last_error()
     pad = _lib.ConvDesc(1, 16, 20, 20, 16, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 16)

@@ -58,6 +58,27 @@ def test_prepared_buffer_int8(dev, K, C, ks):
     assert np.array_equal(buf[frag.size:].view(np.int32), addend)
 
 
+@pytest.mark.parametrize("K,C,kh,kw", [(64, 4, 7, 7), (48, 8, 3, 3), (16, 4, 2, 8), (32, 12, 1, 5)])
+def test_prepared_buffer_int8_c4(dev, K, C, kh, kw):
+    """4-channel blocks: k-step = (channel block, kh), lane -> channel kb * 32 + lane % 32 and taps
+    kw = 4 (lane / 32) .. + 3 (zeros for kw >= KW)."""
+    cc = C // 4
+    wt = rng.uniform_s8((K // 16, cc, kh, kw, 1, 16, 4), K + C)
+    p = U.prepare_conv2d_weight(_t(wt, dev))
+    torch.cuda.synchronize()
+    kblocks, nsteps = (K + 31) // 32, cc * kh
+    w = wt.reshape(K // 16, cc * kh, kw, 16, 4).transpose(0, 3, 1, 2, 4).reshape(K, nsteps, kw, 4)  # [k][ci*KH+kh][kw][ci4]
+    full = np.zeros((kblocks * 32, nsteps, 8, 4), np.int8)
+    full[:K, :, :kw] = w
+    frag = full.reshape(kblocks, 32, nsteps, 2, 16).transpose(0, 2, 3, 1, 4).reshape(kblocks, nsteps, 64, 16)
+    addend = np.zeros(kblocks * 32, np.int32)
+    addend[:K] = 128 * w.astype(np.int64).sum(axis=(1, 2, 3))
+    buf = p.buf.cpu().numpy()
+    assert buf.size == frag.size + addend.size * 4
+    assert np.array_equal(buf[:frag.size].view(np.int8).reshape(frag.shape), frag)
+    assert np.array_equal(buf[frag.size:].view(np.int32), addend)
+
+
 @pytest.mark.parametrize("K,C,ks", [(64, 64, 3), (48, 16, 1), (16, 48, 2)])
 def test_prepared_buffer_fp16(dev, K, C, ks):
     b = rng.normal_f16((K // 16, C // 16, ks, ks, 16, 16), K + C)
@@ -97,6 +118,65 @@ def test_conv2d_prepared_bit_exact(dev, oracle, N, C, H, W, K, ks, stride, pad, 
     assert "prep" in U.last_variant()
     assert tuple(out.shape) == ref.shape
     assert np.array_equal(out.cpu().numpy(), ref), U.last_variant()
+
+
+C4_CASES = [
+    # N, C (padded to 4s), H, W, K, (KH, KW), stride, pad, dilation
+    (1, 4, 32, 32, 64, (7, 7), 2, 3, 1),          # the stem, small
+    (1, 4, 224, 224, 64, (7, 7), 2, 3, 1),        # the stem, full size (apps/cpu/relay/result.log:6803-6828)
+    (2, 8, 11, 13, 16, (3, 3), 1, (0, 1, 2, 1), 1),   # two channel blocks, asymmetric pad
+    (3, 4, 9, 10, 48, (5, 8), (2, 1), (2, 3), 1),     # KW = 8: both halves full; K not a multiple of 32
+    (1, 12, 7, 7, 32, (3, 1), 1, 0, (2, 1)),          # one tap per row, dilation along H, no padding
+    (2, 4, 6, 5, 16, (1, 1), 1, 0, 1),                # 1x1: one k-step
+    (32, 4, 224, 224, 64, (7, 7), 2, 3, 1),           # ResNet-50 batch 32 stem
+]
+
+
+@pytest.mark.parametrize("N,C,H,W,K,ks,stride,pad,dil", C4_CASES)
+def test_conv2d_prepared_c4_bit_exact(dev, oracle, N, C, H, W, K, ks, stride, pad, dil):
+    kh, kw = ks
+    data = rng.uniform_u8((N, C // 4, H, W, 4), 7 * C + H)
+    wt = rng.uniform_s8((K // 16, C // 4, kh, kw, 1, 16, 4), 3 * K + kh)
+    if N == 32:   # the oracle takes its time on the full batch: check two images of it
+        ref = oracle.c_conv2d_nchwc(data[[0, 31]], wt, stride, pad, dil)
+    else:
+        ref = oracle.c_conv2d_nchwc(data, wt, stride, pad, dil)
+    p = U.prepare_conv2d_weight(_t(wt, dev))
+    out = U.conv2d_NCHWc_int8(_t(data, dev), p, stride, pad, dil, "int32", "NCHW4c", "NCHW16c")
+    torch.cuda.synchronize()
+    assert U.last_variant().startswith("i8prep_c4")
+    got = out.cpu().numpy()
+    if N == 32:
+        got = got[[0, 31]]
+    assert got.shape == ref.shape
+    assert np.array_equal(got, ref), U.last_variant()
+    # fused signed form on the same prepared weights
+    xs = (data ^ 0x80).view(np.int8)
+    bias = rng.uniform_s8((K,), 5).astype(np.int32) * 313
+    if N != 32:
+        ref_f = oracle.conv2d_nchwc_int8_fused(xs, wt, bias, 5, stride, pad, dil, conv=oracle.c_conv2d_nchwc)
+        out = U.conv2d_NCHWc_int8_fused(_t(xs, dev), p, _t(bias, dev), 5, stride, pad, dil, "int32", "NCHW4c", "NCHW16c")
+        torch.cuda.synchronize()
+        assert U.last_variant().startswith("s8prep_c4")
+        assert np.array_equal(out.cpu().numpy(), ref_f), U.last_variant()
+
+
+def test_conv2d_prepared_c4_every_direct_variant(dev, oracle, monkeypatch):
+    from unit_amd import _lib
+    N, C, H, W, K = 2, 8, 13, 17, 96
+    data = rng.uniform_u8((N, C // 4, H, W, 4), 21)
+    wt = rng.uniform_s8((K // 16, C // 4, 7, 7, 1, 16, 4), 22)
+    ref = oracle.c_conv2d_nchwc(data, wt, 2, 3, 1)
+    d = _t(data, dev)
+    p = U.prepare_conv2d_weight(_t(wt, dev))
+    names = set()
+    for v in range(1, _lib.load().unit_conv_variant_count() + 1):
+        monkeypatch.setenv("UNIT_AMD_CONV_VARIANT", str(v))
+        out = U.conv2d_NCHWc_int8(d, p, 2, 3, 1, "int32", "NCHW4c")
+        torch.cuda.synchronize()
+        names.add(U.last_variant())
+        assert np.array_equal(out.cpu().numpy(), ref), (v, U.last_variant())
+    assert len(names) >= 15 and all(n.startswith("i8prep_c4") for n in names), names
 
 
 @pytest.mark.parametrize("N,C,H,W,K,ks,stride,pad", [
@@ -195,5 +275,8 @@ def test_prepared_rejections(dev):
         U.conv2d_NCHWc_int8(_t(rng.uniform_u8((1, 3, 8, 8, 16), 2), dev), p, 1, 1)
     with pytest.raises(TypeError):    # int8 weights into the fp16 operator
         U.conv2d_NCHW16c_OHWI16o(_t(rng.normal_f16((1, 2, 8, 8, 16), 3), dev), p, 1, 1)
-    with pytest.raises(ValueError):   # 4-channel blocks have no prepared form
-        U.prepare_conv2d_weight(_t(rng.uniform_s8((2, 1, 3, 3, 1, 16, 4), 1), dev))
+    with pytest.raises(ValueError):   # 4-channel blocks: KW <= 8 only
+        U.prepare_conv2d_weight(_t(rng.uniform_s8((2, 1, 3, 9, 1, 16, 4), 1), dev))
+    with pytest.raises(ValueError):   # prepared for 4-channel blocks, data in 16-channel blocks
+        p4 = U.prepare_conv2d_weight(_t(rng.uniform_s8((2, 4, 3, 3, 1, 16, 4), 1), dev))
+        U.conv2d_NCHWc_int8(_t(rng.uniform_u8((1, 1, 8, 8, 16), 2), dev), p4, 1, 1)

@@ -87,8 +87,8 @@ def load():
     L.unit_prepack_conv_weight_s8.argtypes = [vp, vp, i32, i32, i32, i32, i32, vp]
     L.unit_prepack_dense_weight_s8.argtypes = [vp, vp, i32, i32, vp]
     L.unit_prepack_conv_weight_f16.argtypes = [vp, vp, i32, i32, i32, i32, vp]
-    L.unit_conv2d_prepared_weight_bytes.argtypes = [i32, i32, i32, i32, i32, ctypes.POINTER(ctypes.c_size_t)]
-    L.unit_conv2d_prepare_weight.argtypes = [i32, i32, i32, i32, i32, vp, vp, vp]
+    L.unit_conv2d_prepared_weight_bytes.argtypes = [i32, i32, i32, i32, i32, i32, ctypes.POINTER(ctypes.c_size_t)]
+    L.unit_conv2d_prepare_weight.argtypes = [i32, i32, i32, i32, i32, i32, vp, vp, vp]
     L.unit_conv2d_nchwc_u8s8s32_prepared.argtypes = [dp, vp, vp, vp, vp]
     L.unit_conv2d_nchwc_s8s8s32_fused_prepared.argtypes = [dp, vp, vp, vp, i32, vp, vp]
     L.unit_conv2d_nchw16c_f16f32_prepared.argtypes = [dp, vp, vp, vp, vp]

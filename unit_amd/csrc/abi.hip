@@ -80,6 +80,7 @@ int conv_geom(const unit_conv_desc *d, int tapb, ConvGeom *g, const char *what) 
   g->npix = (int)npix;
   g->ntaps = cc * d->KH * d->KW;
   g->ntab = g->ntaps;
+  g->c4_steps = cc * d->KH;
   g->img_bytes = (u32)img;
   g->by_ohw = FastDiv::make(OH * OW);
   g->by_ow = FastDiv::make(OW);

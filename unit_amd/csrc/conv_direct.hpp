@@ -30,6 +30,13 @@
 // or eight 16-bit loads, and for u8 data the 128 * sum(w) correction is a per-channel constant
 // that prepare_weight left behind the fragments (passed here as the bias), so the reduction loop
 // does not accumulate weight sums.  The fragment that pads an odd tap count is zero.
+//
+// C4 (with PREP, int8): data in 4-channel blocks (N, C/4, H, W, 4), the layout of the 3-channel
+// stem.  A pixel is 4 bytes, so the KW taps of one window row are consecutive memory: a k-step is
+// one row kh of one channel block, lanes 0-31 hold its taps kw = 0..3 and lanes 32-63 kw = 4..7 (KW <= 8,
+// no dilation along W; prepared weights are zero for kw >= KW).  Each tap is its own dword load with
+// its own mask (row inside the image, per k-step; column inside the image and kw < KW, constant per
+// lane), so no load leaves the tensor.
 #pragma once
 #include "epilogues.hpp"
 #include "loaders.hpp"
@@ -102,15 +109,16 @@ __device__ __forceinline__ void store_block(const typename ConvEpilogue<Op>::Par
   }
 }
 
-template <class Op, class S, bool SHIFT, bool PREP = false>
+template <class Op, class S, bool SHIFT, bool PREP = false, bool C4 = false>
 __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ data, const char *__restrict__ wgt,
                                                      typename ConvEpilogue<Op>::Params ep, ConvGeom g, GridMap gm) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   constexpr int TX = S::TX, TY = S::TY, KG = S::KG, D = S::D;
   constexpr bool kInt = Op::kInt;
-  constexpr int TAPB = kInt ? 16 : 32;      // bytes of one pixel and tap
-  constexpr int WTAP = kInt ? 256 : 512;    // bytes of one tap of a 16-channel weight block
+  constexpr int TAPB = C4 ? 4 : (kInt ? 16 : 32);  // bytes of one pixel and tap
+  constexpr int WTAP = kInt ? 256 : 512;           // bytes of one tap of a 16-channel weight block
   static_assert(kInt || (!SHIFT && !S::PAD), "the fp16 operator has neither a shift nor padding");
+  static_assert(!C4 || (kInt && PREP && S::PAD), "4-channel blocks: int8 on prepared weights, masked loads");
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int l32 = lane & 31, half = lane >> 5;
@@ -125,11 +133,17 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
   // tap (ci, kd, kh, kw) -> (byte offset of the tap inside an image relative to the window origin,
   // index of its window position kh * KW + kw).  int8 pairs taps into k-steps: the odd tap past the end points
   // at bit 31 of the window set, which is never set, so it is staged like zero padding.
-  const int nsteps = kInt ? (g.ntaps + 1) >> 1 : g.ntaps;
+  // C4: a k-step is (channel block, kh); the table holds the row's offset for both halves and kh
+  const int nsteps = C4 ? g.c4_steps : (kInt ? (g.ntaps + 1) >> 1 : g.ntaps);
   const int ntab = kInt ? 2 * nsteps : nsteps;
   for (int e = threadIdx.x; e < ntab; e += S::NT) {
     v2i ent = {0, 31};
-    if (e < g.ntaps) {
+    if constexpr (C4) {
+      int ci, kh;
+      g.by_kh.divmod(e >> 1, ci, kh);
+      ent[0] = ((ci * g.H + kh * g.dh) * g.W) * 4 + (e & 1) * 16;
+      ent[1] = g.nopad ? 0 : kh;
+    } else if (e < g.ntaps) {
       int kw, rest, kh, rest2, kd, ci;
       g.by_kw.divmod(e, rest, kw);
       g.by_kh.divmod(rest, rest2, kh);
@@ -176,11 +190,13 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
   // window positions (kh, kw) that fall inside the image (none for lanes past the last pixel)
   int pixoff[TY];
   u32 inside[TY];
+  v4i colm[C4 ? TY : 1];  // C4: per tap of this lane's half, all ones if its column is inside the image and kw < KW
 #pragma unroll
   for (int j = 0; j < TY; ++j) {
     const int m = y0 + j * 32 + l32;
-    pixoff[j] = kInt ? 0 : half * 16;
+    pixoff[j] = (kInt || C4) ? 0 : half * 16;
     inside[j] = 0;
+    if constexpr (C4) colm[j] = v4i{0, 0, 0, 0};
     if (m < g.npix) {
       int n, rem, od, rem2, oh, ow;
       g.by_ohw.divmod(m, n, rem);
@@ -188,7 +204,16 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
       g.by_ow.divmod(rem2, oh, ow);
       const int ih0 = oh * g.sh - g.pt, iw0 = ow * g.sw - g.pl;
       pixoff[j] += (int)(n * g.img_bytes) + ((od * g.sd * g.H + ih0) * g.W + iw0) * TAPB;
-      if constexpr (S::PAD) {
+      if constexpr (C4) {
+        u32 rows = 0;  // rows kh inside the image
+        for (int kh = 0; kh < g.KH; ++kh) rows |= (u32)((u32)(ih0 + kh * g.dh) < (u32)g.H) << kh;
+        inside[j] = g.nopad ? 1u : rows;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int kw = 4 * half + e;
+          colm[j][e] = (kw < g.KW && (u32)(iw0 + kw) < (u32)g.W) ? -1 : 0;
+        }
+      } else if constexpr (S::PAD) {
         u32 cols = 0, bits = 0;  // columns kw inside the image; then one copy of them per row kh inside
         for (int kw = 0; kw < g.KW; ++kw) cols |= (u32)((u32)(iw0 + kw * g.dw) < (u32)g.W) << kw;
         for (int kh = 0; kh < g.KH; ++kh)
@@ -211,7 +236,8 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
 
   // prefetch ring: D k-steps of fragments in registers
   v4i xf[D][TX], yf[D][TY];
-  int ym[S::PAD ? D : 1][TY];  // all ones where the tap lies inside the image, else 0
+  int ym[S::PAD && !C4 ? D : 1][TY];  // all ones where the tap lies inside the image, else 0
+  v4i ym4[C4 ? D : 1][TY];           // C4: the same per tap of the fragment
   const u32 last_tap_off = (u32)(g.ntaps - 1) * (u32)WTAP;
 
   // Fetches run through the k-steps in order; `sf` is the next one (it stops at the wave's last
@@ -250,7 +276,17 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
     }
 #pragma unroll
     for (int j = 0; j < TY; ++j) {
-      if constexpr (S::PAD) {
+      if constexpr (C4) {
+        const int rowm = __builtin_amdgcn_sbfe((int)inside[j], (u32)e[1], 1u);
+        const u32 o = (u32)(pixoff[j] + e[0]);
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          const int m = rowm & colm[j][d];
+          // the sum is formed in 32 bits before masking: o alone may lie before the tensor (left edge of row 0)
+          yf[U][j][d] = *reinterpret_cast<const int *>(data + ((o + (u32)(d * 4)) & (u32)m));
+          ym4[U][j][d] = m;
+        }
+      } else if constexpr (S::PAD) {
         // all ones if window position e[1] of this lane's pixel is inside the image, else 0
         const int m = __builtin_amdgcn_sbfe((int)inside[j], (u32)e[1], 1u);
         yf[U][j] = *reinterpret_cast<const v4i *>(data + ((u32)(pixoff[j] + e[0]) & (u32)m));
@@ -268,7 +304,10 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
 #pragma unroll
       for (int d = 0; d < 4; ++d) {
         int v = yf[U][j][d];
-        if constexpr (S::PAD) v &= ym[U][j];
+        if constexpr (C4)
+          v &= ym4[U][j][d];
+        else if constexpr (S::PAD)
+          v &= ym[U][j];
         if constexpr (SHIFT) v ^= (int)0x80808080;
         y[j][d] = v;
       }

@@ -15,6 +15,8 @@ int conv_u8_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGe
                      const int *addend, void *out, hipStream_t s);  // conv_prepared_u8.hip
 int conv_s8_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
                      const int *bias, int scale, void *out, hipStream_t s);  // conv_prepared_s8.hip
+int conv_c4_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
+                     const int *addend, int scale, bool shift, void *out, hipStream_t s);  // conv_prepared_c4.hip
 int conv_f16_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *a, const void *w,
                       void *out, hipStream_t s);  // conv_prepared_f16.hip
 
@@ -34,17 +36,37 @@ __global__ __launch_bounds__(64) void prepare_i8(const char *__restrict__ w, cha
   *reinterpret_cast<v4i *>(out + ((size_t)blk * 64 + lane) * 16) = v;
 }
 
-// one wave per output channel: 128 * sum of its weights
+// 4-channel blocks (K/16, C/4, KH, KW, 1, 16, 4): one workgroup per (32-channel block, ci * KH + kh),
+// a lane gathers 4 consecutive taps of the row (zeros for kw >= KW)
+__global__ __launch_bounds__(64) void prepare_i8_c4(const char *__restrict__ w, char *__restrict__ out, int K, int KH,
+                                                    int KW, int nsteps) {
+  const int blk = blockIdx.x, kb = blk / nsteps, s = blk - kb * nsteps;
+  const int lane = threadIdx.x, ko = kb * 32 + (lane & 31), half = lane >> 5;
+  const int cc = nsteps / KH;
+  v4i v = {0, 0, 0, 0};
+  if (ko < K) {
+    const char *row = w + ((size_t)(ko >> 4) * cc * KH + s) * KW * 64 + (ko & 15) * 4;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int kw = 4 * half + e;
+      if (kw < KW) v[e] = *reinterpret_cast<const int *>(row + kw * 64);
+    }
+  }
+  *reinterpret_cast<v4i *>(out + ((size_t)blk * 64 + lane) * 16) = v;
+}
+
+// one wave per output channel: 128 * sum of its weights (a tap of a 16-output-channel block is
+// `dwords` dwords per channel, 64 bytes apart)
 __global__ __launch_bounds__(64) void prepare_i8_addend(const char *__restrict__ w, int *__restrict__ addend, int K,
-                                                        int ntaps) {
+                                                        int ntaps, int dwords) {
   const int ko = blockIdx.x, lane = threadIdx.x;
   int sum = 0;
   if (ko < K) {
-    const char *src = w + (size_t)(ko >> 4) * ntaps * 256 + (ko & 15) * 4;
+    const size_t tapb = (size_t)dwords * 64;
+    const char *src = w + (size_t)(ko >> 4) * ntaps * tapb + (ko & 15) * 4;
     for (int t = lane; t < ntaps; t += 64)
-#pragma unroll
-      for (int d = 0; d < 4; ++d)
-        sum = __builtin_amdgcn_sdot4(*reinterpret_cast<const int *>(src + (size_t)t * 256 + d * 64), 0x01010101, sum, false);
+      for (int d = 0; d < dwords; ++d)
+        sum = __builtin_amdgcn_sdot4(*reinterpret_cast<const int *>(src + t * tapb + d * 64), 0x01010101, sum, false);
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
@@ -65,12 +87,15 @@ __global__ __launch_bounds__(64) void prepare_f16(const char *__restrict__ w, ch
   *reinterpret_cast<v8h *>(out + ((size_t)blk * 64 + lane) * 16) = h;
 }
 
-int check_weight_shape(const char *what, int K, int C, int KH, int KW, int elem_bytes, PreparedLayout *pl) {
+int check_weight_shape(const char *what, int K, int C, int KH, int KW, int cb, int elem_bytes, PreparedLayout *pl) {
   if (elem_bytes != 1 && elem_bytes != 2) return fail(UNIT_E_ARG, "%s: elem_bytes must be 1 (int8) or 2 (fp16), got %d", what, elem_bytes);
+  if (cb != 16 && !(cb == 4 && elem_bytes == 1))
+    return fail(UNIT_E_ARG, "%s: cb must be 16, or 4 for int8 (got %d)", what, cb);
   if (K <= 0 || C <= 0 || KH <= 0 || KW <= 0) return fail(UNIT_E_ARG, "%s: K, C, KH, KW must be positive", what);
-  if (K % 16 || C % 16) return fail(UNIT_E_ARG, "%s: K and C must be multiples of 16 (got %d, %d)", what, K, C);
+  if (K % 16 || C % cb) return fail(UNIT_E_ARG, "%s: K must be a multiple of 16 and C of cb (got %d, %d)", what, K, C);
+  if (cb == 4 && KW > 8) return fail(UNIT_E_ARG, "%s: 4-channel blocks have a prepared form for KW <= 8 (got %d)", what, KW);
   if (!fits((size_t)K * C * KH * KW * elem_bytes)) return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
-  *pl = prepared_layout(K, C, KH, KW, elem_bytes);
+  *pl = prepared_layout(K, C, KH, KW, cb, elem_bytes);
   if (!fits(pl->total_bytes)) return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
   return UNIT_OK;
 }
@@ -96,7 +121,13 @@ ConvPlan plan_prepared(const unit_conv_desc *d, const ConvGeom &g, int kbytes, c
 }
 
 int check_prepared_conv(const char *what, const unit_conv_desc *d, int tapb, ConvGeom *g) {
-  if (d->cb != 16) return fail(UNIT_E_ARG, "%s: prepared weights serve 16-channel blocks (got cb = %d)", what, d->cb);
+  if (d->cb != 16 && !(d->cb == 4 && tapb == 16))
+    return fail(UNIT_E_ARG, "%s: cb must be 16, or 4 for int8 (got %d)", what, d->cb);
+  if (d->cb == 4) {
+    if (d->KW > 8 || d->KH > 31 || d->dw != 1)
+      return fail(UNIT_E_ARG, "%s: 4-channel blocks need KW <= 8, KH <= 31 and no dilation along W", what);
+    tapb = 4;
+  }
   if (int rc = conv_geom(d, tapb, g, what)) return rc;
   if (tapb == 16 && d->KH * d->KW > 31) return fail(UNIT_E_ARG, "%s: window of %d x %d exceeds 31 positions", what, d->KH, d->KW);
   if (!fits((size_t)g->npix * d->K * 4)) return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
@@ -106,39 +137,42 @@ int check_prepared_conv(const char *what, const unit_conv_desc *d, int tapb, Con
 }  // namespace
 }  // namespace unit
 
-extern "C" int unit_conv2d_prepared_weight_bytes(int32_t K, int32_t C, int32_t KH, int32_t KW, int32_t elem_bytes,
-                                                 size_t *bytes) {
+extern "C" int unit_conv2d_prepared_weight_bytes(int32_t K, int32_t C, int32_t KH, int32_t KW, int32_t cb,
+                                                 int32_t elem_bytes, size_t *bytes) {
   using namespace unit;
   const char *what = "unit_conv2d_prepared_weight_bytes";
   if (!bytes) return fail(UNIT_E_ARG, "%s: null pointer", what);
   PreparedLayout pl;
-  if (int rc = check_weight_shape(what, K, C, KH, KW, elem_bytes, &pl)) return rc;
+  if (int rc = check_weight_shape(what, K, C, KH, KW, cb, elem_bytes, &pl)) return rc;
   *bytes = pl.total_bytes;
   return UNIT_OK;
 }
 
-extern "C" int unit_conv2d_prepare_weight(int32_t K, int32_t C, int32_t KH, int32_t KW, int32_t elem_bytes,
+extern "C" int unit_conv2d_prepare_weight(int32_t K, int32_t C, int32_t KH, int32_t KW, int32_t cb, int32_t elem_bytes,
                                           const void *weight, void *prepared, unit_stream_t stream) {
   using namespace unit;
   const char *what = "unit_conv2d_prepare_weight";
   if (!weight || !prepared) return fail(UNIT_E_ARG, "%s: null pointer", what);
   PreparedLayout pl;
-  if (int rc = check_weight_shape(what, K, C, KH, KW, elem_bytes, &pl)) return rc;
+  if (int rc = check_weight_shape(what, K, C, KH, KW, cb, elem_bytes, &pl)) return rc;
   if (int rc = check_device()) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int ntaps = (C / 16) * KH * KW;
+  const int ntaps = (C / cb) * KH * KW;
   const char *w = static_cast<const char *>(weight);
   char *out = static_cast<char *>(prepared);
   if (elem_bytes == 1) {
-    hipLaunchKernelGGL(prepare_i8, dim3(pl.kblocks * pl.nsteps), dim3(64), 0, s, w, out, K, ntaps, pl.nsteps);
+    if (cb == 4)
+      hipLaunchKernelGGL(prepare_i8_c4, dim3(pl.kblocks * pl.nsteps), dim3(64), 0, s, w, out, K, KH, KW, pl.nsteps);
+    else
+      hipLaunchKernelGGL(prepare_i8, dim3(pl.kblocks * pl.nsteps), dim3(64), 0, s, w, out, K, ntaps, pl.nsteps);
     hipLaunchKernelGGL(prepare_i8_addend, dim3(pl.kblocks * 32), dim3(64), 0, s, w,
-                       reinterpret_cast<int *>(out + pl.frag_bytes), K, ntaps);
+                       reinterpret_cast<int *>(out + pl.frag_bytes), K, ntaps, cb / 4);
   } else {
     hipLaunchKernelGGL(prepare_f16, dim3(pl.kblocks * pl.nsteps), dim3(64), 0, s, w, out, K, ntaps);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "%s: launch: %s", what, hipGetErrorString(e));
-  set_variant("prepare_%s_k%d_s%d", elem_bytes == 1 ? "i8" : "f16", pl.kblocks, pl.nsteps);
+  set_variant("prepare_%s_k%d_s%d", elem_bytes == 2 ? "f16" : (cb == 4 ? "i8c4" : "i8"), pl.kblocks, pl.nsteps);
   return UNIT_OK;
 }
 
@@ -149,12 +183,14 @@ extern "C" int unit_conv2d_nchwc_u8s8s32_prepared(const unit_conv_desc *d, const
   if (!d || !data || !prepared || !out) return fail(UNIT_E_ARG, "%s: null pointer", what);
   ConvGeom g;
   if (int rc = check_prepared_conv(what, d, 16, &g)) return rc;
-  const PreparedLayout pl = prepared_layout(d->K, d->C, d->KH, d->KW, 1);
+  const PreparedLayout pl = prepared_layout(d->K, d->C, d->KH, d->KW, d->cb, 1);
   const int ntable = (int)(sizeof(kTunedI8Prepared) / sizeof(kTunedI8Prepared[0])) - 1;
-  const ConvPlan p = plan_prepared(d, g, g.ntaps * 16, kTunedI8Prepared, ntable, true);
+  const ConvPlan p = plan_prepared(d, g, g.ntaps * d->cb, kTunedI8Prepared, ntable, true);
   const char *w = static_cast<const char *>(prepared);
-  return conv_u8_prepared(p, d, g, data, w, reinterpret_cast<const int *>(w + pl.frag_bytes), out,
-                          static_cast<hipStream_t>(stream));
+  const int *addend = reinterpret_cast<const int *>(w + pl.frag_bytes);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (d->cb == 4) return conv_c4_prepared(p, d, g, data, w, addend, 1, true, out, s);
+  return conv_u8_prepared(p, d, g, data, w, addend, out, s);
 }
 
 extern "C" int unit_conv2d_nchwc_s8s8s32_fused_prepared(const unit_conv_desc *d, const void *data,
@@ -166,8 +202,10 @@ extern "C" int unit_conv2d_nchwc_s8s8s32_fused_prepared(const unit_conv_desc *d,
   ConvGeom g;
   if (int rc = check_prepared_conv(what, d, 16, &g)) return rc;
   const int ntable = (int)(sizeof(kTunedI8Prepared) / sizeof(kTunedI8Prepared[0])) - 1;
-  const ConvPlan p = plan_prepared(d, g, g.ntaps * 16, kTunedI8Prepared, ntable, true);
-  return conv_s8_prepared(p, d, g, data, prepared, bias, scale, out, static_cast<hipStream_t>(stream));
+  const ConvPlan p = plan_prepared(d, g, g.ntaps * d->cb, kTunedI8Prepared, ntable, true);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (d->cb == 4) return conv_c4_prepared(p, d, g, data, prepared, bias, scale, false, out, s);
+  return conv_s8_prepared(p, d, g, data, prepared, bias, scale, out, s);
 }
 
 extern "C" int unit_conv2d_nchw16c_f16f32_prepared(const unit_conv_desc *d, const void *a, const void *prepared,

@@ -2,8 +2,10 @@
 // load per lane and k-step (conv_direct.hpp, PREP).
 //
 //   prepared[kb][s][lane][16 bytes], kb = 32-channel block of K, s = k-step, lane = 0..63:
-//     int8: channel kb * 32 + lane % 32, tap 2 s + lane / 32 (taps run (ci, kh, kw) as in the
-//           reference's (K/16, C/16, KH, KW, 4, 16, 4) layout), its 16 input channels;
+//     int8, 16-channel blocks: channel kb * 32 + lane % 32, tap 2 s + lane / 32 (taps run (ci, kh, kw)
+//           as in the reference's (K/16, C/16, KH, KW, 4, 16, 4) layout), its 16 input channels;
+//     int8, 4-channel blocks (K/16, C/4, KH, KW, 1, 16, 4): k-step s = ci * KH + kh is one window row,
+//           the lane holds taps kw = 4 (lane / 32) .. + 3 of it, 4 input channels each (KW <= 8);
 //     fp16: channel kb * 32 + lane % 32, tap s, input channels 8 (lane / 32) .. + 8;
 //   channels past K and the tap that pads an odd tap count are zeros;
 //   int8 only, behind the fragments: int32 addend[kb * 32 + c] = 128 * sum of the channel's weights
@@ -19,11 +21,11 @@ struct PreparedLayout {
   size_t total_bytes;   // + the addends for int8
 };
 
-inline PreparedLayout prepared_layout(int K, int C, int KH, int KW, int elem_bytes) {
+inline PreparedLayout prepared_layout(int K, int C, int KH, int KW, int cb, int elem_bytes) {
   PreparedLayout p;
-  const int ntaps = (C / 16) * KH * KW;
+  const int ntaps = (C / cb) * KH * KW;
   p.kblocks = (K + 31) / 32;
-  p.nsteps = elem_bytes == 1 ? (ntaps + 1) / 2 : ntaps;
+  p.nsteps = cb == 4 ? (C / 4) * KH : (elem_bytes == 1 ? (ntaps + 1) / 2 : ntaps);
   p.frag_bytes = (size_t)p.kblocks * p.nsteps * 1024;
   p.total_bytes = p.frag_bytes + (elem_bytes == 1 ? (size_t)p.kblocks * 32 * 4 : 0);
   return p;

@@ -236,6 +236,7 @@ struct ConvGeom {
   int npix;    // N * OH * OW
   int ntaps;   // (C / cb) * KH * KW
   int ntab;    // table entries (ntaps rounded up to whole pipeline stages)
+  int c4_steps;  // (C / 4) * KH: k-steps of the direct kernel on 4-channel blocks (one window row each)
   u32 img_bytes;  // bytes per image
   FastDiv by_ohw, by_ow, by_kh, by_kw;  // dividers by output pixels per image, OW, KH, KW
   // depth, for the 3-D convolution (direct kernels only); 1 / 1 / 1 / 1 for 2-D, where

@@ -94,11 +94,12 @@ class PreparedConvWeight:
     Accepted wherever conv2d_NCHWc_int8, conv2d_NCHWc_int8_fused and conv2d_NCHW16c_OHWI16o take
     a kernel."""
 
-    def __init__(self, buf, K, C, KH, KW, dtype):
-        self.buf, self.K, self.C, self.KH, self.KW, self.dtype = buf, K, C, KH, KW, dtype
+    def __init__(self, buf, K, C, KH, KW, cb, dtype):
+        self.buf, self.K, self.C, self.KH, self.KW, self.cb, self.dtype = buf, K, C, KH, KW, cb, dtype
 
     def __repr__(self):
-        return f"PreparedConvWeight(K={self.K}, C={self.C}, KH={self.KH}, KW={self.KW}, dtype={self.dtype})"
+        return (f"PreparedConvWeight(K={self.K}, C={self.C}, KH={self.KH}, KW={self.KW}, cb={self.cb}, "
+                f"dtype={self.dtype})")
 
 
 def prepare_conv2d_weight(kernel):
@@ -106,7 +107,8 @@ def prepare_conv2d_weight(kernel):
     constant sub-graphs the reference's compiled models keep next to each convolution (weight
     layout chain apps/cpu/relay/result.log:8-13, sum(w) result.log:15-16).
 
-    kernel int8 (K/16, C/16, KH, KW, 4, 16, 4) or fp16 (K/16, C/16, KH, KW, 16 in, 16 out)
+    kernel int8 (K/16, C/16, KH, KW, 4, 16, 4), int8 (K/16, C/4, KH, KW, 1, 16, 4) with KW <= 8 (the stem's
+           4-channel blocks), or fp16 (K/16, C/16, KH, KW, 16 in, 16 out)
     returns a PreparedConvWeight; convolutions on it give the same results as on `kernel`.
     """
     import ctypes
@@ -115,19 +117,19 @@ def prepare_conv2d_weight(kernel):
         ko, cc, kh, kw, ic, ob = kernel.shape
         if (ic, ob) != (16, 16):
             raise ValueError(f"kernel: expected (K/16, C/16, KH, KW, 16, 16), got {tuple(kernel.shape)}")
-        eb = 2
+        eb, cb = 2, 16
     else:
         kernel = _dev(kernel, "kernel", torch.int8, 7)
         ko, cc, kh, kw, e, kb, i4 = kernel.shape
-        if (e, kb, i4) != (4, 16, 4):
-            raise ValueError(f"kernel: expected (K/16, C/16, KH, KW, 4, 16, 4), got {tuple(kernel.shape)}")
-        eb = 1
+        if e not in (1, 4) or (kb, i4) != (16, 4):
+            raise ValueError(f"kernel: expected (K/16, C/cb, KH, KW, cb/4, 16, 4) with cb 16 or 4, got {tuple(kernel.shape)}")
+        eb, cb = 1, 4 * e
     L = _lib.load()
     nbytes = ctypes.c_size_t()
-    check(L.unit_conv2d_prepared_weight_bytes(ko * 16, cc * 16, kh, kw, eb, ctypes.byref(nbytes)))
+    check(L.unit_conv2d_prepared_weight_bytes(ko * 16, cc * cb, kh, kw, cb, eb, ctypes.byref(nbytes)))
     buf = torch.empty(nbytes.value, dtype=torch.uint8, device=kernel.device)
-    check(L.unit_conv2d_prepare_weight(ko * 16, cc * 16, kh, kw, eb, kernel.data_ptr(), buf.data_ptr(), _stream()))
-    return PreparedConvWeight(buf, ko * 16, cc * 16, kh, kw, kernel.dtype)
+    check(L.unit_conv2d_prepare_weight(ko * 16, cc * cb, kh, kw, cb, eb, kernel.data_ptr(), buf.data_ptr(), _stream()))
+    return PreparedConvWeight(buf, ko * 16, cc * cb, kh, kw, cb, kernel.dtype)
 
 
 def _prepared_dims(kernel, data, want_dtype):
@@ -135,8 +137,8 @@ def _prepared_dims(kernel, data, want_dtype):
     n, cc, h, w, cb = data.shape
     if kernel.dtype != want_dtype:
         raise TypeError(f"kernel: prepared from {kernel.dtype}, this operator takes {want_dtype}")
-    if cb != 16 or kernel.C != cc * 16:
-        raise ValueError(f"kernel: {kernel!r} does not match data {tuple(data.shape)} (16-channel blocks only)")
+    if cb != kernel.cb or kernel.C != cc * cb:
+        raise ValueError(f"kernel: {kernel!r} does not match data {tuple(data.shape)}")
     if kernel.buf.device != data.device:
         raise ValueError("kernel: prepared on another device")
     return kernel.K // 16, cc, kernel.KH, kernel.KW

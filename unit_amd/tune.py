@@ -7,7 +7,7 @@ Here the candidates are the tile variants compiled into libunit_amd.so.  For eve
 each variant is run through the C ABI, checked bit for bit against the library's default choice,
 and timed with HIP events; the fastest goes into unit_amd/csrc/tuned_conv_{i8,f16}.inc, which the
 library's planner consults first (rebuild after tuning).  Needs an MI355X.  With --prepared the
-convolutions on prepared weights are tuned (direct variants only, 16-channel blocks only) into
+convolutions on prepared weights are tuned (direct variants only) into
 tuned_conv_{i8,f16}_prepared.inc.
 
     python -m unit_amd.tune [--dtype i8|f16] [--prepared] [--nets resnet50:32,resnet18:1] [--iters 20] [--write]
@@ -66,7 +66,7 @@ def tune(spec, iters=20, verbose=True, dtype="i8", prepared=False):
             cb = WL.channel_block(s.C) if dtype == "i8" else 16
             if s.C % cb and dtype != "i8":
                 continue  # the fp16 operator needs C % 16 == 0
-            if prepared and (cb != 16 or (dtype == "i8" and s.KH * s.KW > 31)):
+            if prepared and ((cb == 16 and dtype == "i8" and s.KH * s.KW > 31) or (cb == 4 and s.KW > 8)):
                 continue  # no prepared form
             cp = -(-s.C // cb) * cb
             oh, ow = WL.out_hw(s)
