@@ -173,6 +173,11 @@ int unit_prepack_dense_weight_s8(const void *src, void *dst, int32_t N, int32_t 
 int unit_prepack_conv_weight_f16(const void *src, void *dst, int32_t O, int32_t I, int32_t KH,
                                  int32_t KW, unit_stream_t stream);
 
+/* Alignment: every tensor pointer passed to a convolution, dense, GEMM or prepare entry point
+ * must be 16-byte aligned (the kernels use 16-byte vector accesses); a misaligned one is
+ * rejected with UNIT_E_ARG.  Framework allocations (256 bytes and up) satisfy this; a view that
+ * starts inside an allocation may not. */
+
 /* ------------------------------------------------------------------ prepared weights */
 
 /* Convolution weights re-ordered once into the MFMA fragment order of the kernels, with the

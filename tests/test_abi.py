@@ -100,6 +100,13 @@ def test_out_hw_and_error_paths_without_gpu():
     assert L.unit_conv2d_nchwc_s8s8s32_fused_prepared(ctypes.byref(big), 1, 1, None, 1, 1, None) == -1 and b"31 positions" in L.unit_last_error()
     pad = _lib.ConvDesc(1, 16, 20, 20, 16, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 16)
     assert L.unit_conv2d_nchw16c_f16f32_prepared(ctypes.byref(pad), 1, 1, 1, None) == -1 and b"padding" in L.unit_last_error()
+    # tensor pointers must be 16-byte aligned (the kernels use 16-byte vector accesses)
+    ok = _lib.ConvDesc(1, 16, 8, 8, 16, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 16)
+    for args in ((8, 16, 16), (16, 4, 16), (16, 16, 24)):
+        assert L.unit_conv2d_nchwc_u8s8s32(ctypes.byref(ok), *args, None) == -1 and b"aligned" in L.unit_last_error()
+        assert L.unit_conv2d_nchwc_u8s8s32_prepared(ctypes.byref(ok), *args, None) == -1 and b"aligned" in L.unit_last_error()
+    assert L.unit_dense_u8s8s32(16, 16, 8, 16, 16, 16, None) == -1 and b"aligned" in L.unit_last_error()
+    assert L.unit_gemm_f16(16, 2, 16, 16, 16, 16, 0, None) == -1 and b"aligned" in L.unit_last_error()
     # size limit: every tensor must stay below 2^31 bytes (32-bit offsets in the kernels)
     huge = _lib.ConvDesc(4096, 256, 56, 56, 256, 1, 1, 1, 1, 0, 0, 0, 0, 1, 1, 16)
     assert L.unit_conv2d_nchwc_u8s8s32(ctypes.byref(huge), 1, 1, 1, None) == -1 and b"2^31" in L.unit_last_error()

@@ -268,6 +268,19 @@ def test_conv2d_fp16_prepared_every_direct_variant(dev, oracle, monkeypatch):
     assert len(names) >= 15 and all(n.startswith("f16prep") for n in names), names
 
 
+def test_misaligned_views_are_rejected(dev):
+    """A tensor view that starts 8 bytes into an allocation: the library refuses it instead of issuing
+    misaligned 16-byte accesses."""
+    flat = _t(rng.uniform_u8((1 * 2 * 8 * 8 * 16 + 8,), 3), dev)
+    data = flat[8:].view(1, 2, 8, 8, 16)
+    assert data.data_ptr() % 16 == 8
+    wt = _t(rng.uniform_s8((2, 2, 3, 3, 4, 16, 4), 1), dev)
+    with pytest.raises(ValueError, match="aligned"):
+        U.conv2d_NCHWc_int8(data, wt, 1, 1)
+    with pytest.raises(ValueError, match="aligned"):
+        U.conv2d_NCHWc_int8(data, U.prepare_conv2d_weight(wt), 1, 1)
+
+
 def test_prepared_rejections(dev):
     wt = _t(rng.uniform_s8((2, 2, 3, 3, 4, 16, 4), 1), dev)
     p = U.prepare_conv2d_weight(wt)

@@ -26,6 +26,7 @@ extern "C" int unit_conv3d_ncdhwc_s8s8s32(const unit_conv3d_desc *d, const void 
   const size_t taps = (size_t)cc * d->KD * d->KH * d->KW;
   if (!fits(img * d->N) || npix > kMaxTensorBytes || !fits((size_t)d->K * taps * 16) || !fits(npix * d->K * 4))
     return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
+  if (int rc = check_aligned(what, {data, weight, out})) return rc;
   if (int rc = check_device()) return rc;
   ConvGeom g;
   g.N = d->N; g.H = d->H; g.W = d->W; g.OH = OH; g.OW = OW;

@@ -71,6 +71,7 @@ extern "C" int unit_conv2d_nchw16c_f16f32(const unit_conv_desc *d, const void *a
   ConvGeom g;
   if (int rc = conv_geom(d, 32, &g, what)) return rc;
   if (!fits((size_t)g.npix * d->K * 4)) return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
+  if (int rc = check_aligned(what, {a, b, out})) return rc;
   if (int rc = check_device()) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int ntable = (int)(sizeof(kTunedF16) / sizeof(kTunedF16[0])) - 1;

@@ -42,6 +42,7 @@ extern "C" int unit_conv2d_nchwc_u8s8s32(const unit_conv_desc *d, const void *da
   ConvGeom g;
   if (int rc = conv_geom(d, d->cb, &g, what)) return rc;
   if (!fits((size_t)g.npix * d->K * 4)) return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
+  if (int rc = check_aligned(what, {data, weight, out})) return rc;
   if (int rc = check_device()) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int ntable = (int)(sizeof(kTunedI8) / sizeof(kTunedI8[0])) - 1;

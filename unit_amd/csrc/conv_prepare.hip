@@ -120,7 +120,8 @@ ConvPlan plan_prepared(const unit_conv_desc *d, const ConvGeom &g, int kbytes, c
   return p;
 }
 
-int check_prepared_conv(const char *what, const unit_conv_desc *d, int tapb, ConvGeom *g) {
+int check_prepared_conv(const char *what, const unit_conv_desc *d, int tapb, ConvGeom *g, const void *data,
+                        const void *prepared, const void *out) {
   if (d->cb != 16 && !(d->cb == 4 && tapb == 16))
     return fail(UNIT_E_ARG, "%s: cb must be 16, or 4 for int8 (got %d)", what, d->cb);
   if (d->cb == 4) {
@@ -131,6 +132,7 @@ int check_prepared_conv(const char *what, const unit_conv_desc *d, int tapb, Con
   if (int rc = conv_geom(d, tapb, g, what)) return rc;
   if (tapb == 16 && d->KH * d->KW > 31) return fail(UNIT_E_ARG, "%s: window of %d x %d exceeds 31 positions", what, d->KH, d->KW);
   if (!fits((size_t)g->npix * d->K * 4)) return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
+  if (int rc = check_aligned(what, {data, prepared, out})) return rc;
   return check_device();
 }
 
@@ -155,6 +157,7 @@ extern "C" int unit_conv2d_prepare_weight(int32_t K, int32_t C, int32_t KH, int3
   if (!weight || !prepared) return fail(UNIT_E_ARG, "%s: null pointer", what);
   PreparedLayout pl;
   if (int rc = check_weight_shape(what, K, C, KH, KW, cb, elem_bytes, &pl)) return rc;
+  if (int rc = check_aligned(what, {weight, prepared})) return rc;
   if (int rc = check_device()) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int ntaps = (C / cb) * KH * KW;
@@ -182,7 +185,7 @@ extern "C" int unit_conv2d_nchwc_u8s8s32_prepared(const unit_conv_desc *d, const
   const char *what = "unit_conv2d_nchwc_u8s8s32_prepared";
   if (!d || !data || !prepared || !out) return fail(UNIT_E_ARG, "%s: null pointer", what);
   ConvGeom g;
-  if (int rc = check_prepared_conv(what, d, 16, &g)) return rc;
+  if (int rc = check_prepared_conv(what, d, 16, &g, data, prepared, out)) return rc;
   const PreparedLayout pl = prepared_layout(d->K, d->C, d->KH, d->KW, d->cb, 1);
   const int ntable = (int)(sizeof(kTunedI8Prepared) / sizeof(kTunedI8Prepared[0])) - 1;
   const ConvPlan p = plan_prepared(d, g, g.ntaps * d->cb, kTunedI8Prepared, ntable, true);
@@ -200,7 +203,7 @@ extern "C" int unit_conv2d_nchwc_s8s8s32_fused_prepared(const unit_conv_desc *d,
   const char *what = "unit_conv2d_nchwc_s8s8s32_fused_prepared";
   if (!d || !data || !prepared || !out) return fail(UNIT_E_ARG, "%s: null pointer", what);
   ConvGeom g;
-  if (int rc = check_prepared_conv(what, d, 16, &g)) return rc;
+  if (int rc = check_prepared_conv(what, d, 16, &g, data, prepared, out)) return rc;
   const int ntable = (int)(sizeof(kTunedI8Prepared) / sizeof(kTunedI8Prepared[0])) - 1;
   const ConvPlan p = plan_prepared(d, g, g.ntaps * d->cb, kTunedI8Prepared, ntable, true);
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -216,7 +219,7 @@ extern "C" int unit_conv2d_nchw16c_f16f32_prepared(const unit_conv_desc *d, cons
   if (d->pt || d->pl || d->pb || d->pr) return fail(UNIT_E_ARG, "%s: the operator has no padding argument; pre-pad the data", what);
   if (d->dh != 1 || d->dw != 1) return fail(UNIT_E_ARG, "%s: dilation must be 1", what);
   ConvGeom g;
-  if (int rc = check_prepared_conv(what, d, 32, &g)) return rc;
+  if (int rc = check_prepared_conv(what, d, 32, &g, a, prepared, out)) return rc;
   const int ntable = (int)(sizeof(kTunedF16Prepared) / sizeof(kTunedF16Prepared[0])) - 1;
   const ConvPlan p = plan_prepared(d, g, g.ntaps * 32, kTunedF16Prepared, ntable, false);
   return conv_f16_prepared(p, d, g, a, prepared, out, static_cast<hipStream_t>(stream));

@@ -57,6 +57,7 @@ extern "C" int unit_conv2d_nchwc_s8s8s32_fused(const unit_conv_desc *d, const vo
   ConvGeom g;
   if (int rc = conv_geom(d, d->cb, &g, kWhat)) return rc;
   if (!fits((size_t)g.npix * d->K * 4)) return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", kWhat);
+  if (int rc = check_aligned(kWhat, {data, weight, out})) return rc;
   if (int rc = check_device()) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (d->cb == 16 && d->KH * d->KW <= 31) {

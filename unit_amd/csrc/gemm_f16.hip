@@ -51,6 +51,7 @@ extern "C" int unit_gemm_f16(const void *a, const void *b, void *c, int32_t M, i
   if (N % 4) return fail(UNIT_E_ARG, "%s: N must be a multiple of 4 (got %d)", what, N);
   if (!fits((size_t)M * K * 2) || !fits((size_t)N * K * 2) || !fits((size_t)M * N * 4))
     return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
+  if (int rc = check_aligned(what, {a, b, c})) return rc;
   if (int rc = check_device()) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   return out_f16 ? gemm_f16<true>(a, b, c, M, N, K, s) : gemm_f16<false>(a, b, c, M, N, K, s);

@@ -98,6 +98,7 @@ int dense(const void *a, const void *w, void *c, int M, int N, int K, unit_strea
   if (!PACKED && N % 4) return fail(UNIT_E_ARG, "%s: N must be a multiple of 4 (got %d)", what, N);
   if (!fits((size_t)M * K) || !fits((size_t)N * K) || !fits((size_t)M * N * 4))
     return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
+  if (int rc = check_aligned(what, {a, w, c})) return rc;
   if (int rc = check_device()) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const long tiles_big = (long)ceil_div(M, 256) * ceil_div(N, 256);

@@ -6,6 +6,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <initializer_list>
+
 #include "../../include/unit_amd.h"
 #include "mma_core.hpp"
 
@@ -42,6 +44,15 @@ constexpr int kMaxLds = 160 * 1024;
 inline bool fits(size_t bytes) { return bytes <= kMaxTensorBytes; }
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// The kernels move operands and results with 16-byte vector accesses: every tensor pointer handed
+// to a compute entry point must be 16-byte aligned (framework allocators give 256 bytes or more).
+inline int check_aligned(const char *what, std::initializer_list<const void *> ptrs) {
+  for (const void *p : ptrs)
+    if (reinterpret_cast<uintptr_t>(p) % 16)
+      return fail(UNIT_E_ARG, "%s: tensor pointers must be 16-byte aligned (got %p)", what, p);
+  return UNIT_OK;
+}
 
 // Enqueue mma_kernel over gx x gy tiles and `splits` k-ranges.  With splits > 1 the epilogue
 // accumulates with atomics, so `out` (out_bytes, a multiple of 16) is zero-filled first.
