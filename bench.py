@@ -316,14 +316,15 @@ def main():
         _, fr_us, _ = conv_i8_leg(WL.RESNET50, BATCH, 20, fused=True)
         fused_s8["reference_layout_weights_stack_us"] = round(fr_us, 1)
 
-    # 3-D convolution workloads of apps/cpu/kernel/conv3d.py:13-25 (depth 16, batch 1; the 4-channel one left out)
+    # 3-D convolution workloads of apps/cpu/kernel/conv3d.py:13-25 (depth 16, batch 1)
     c3_rows = []
     for i, (ic, h, w_, oc, ks, st) in enumerate(((256, 16, 16, 256, 3, 1), (512, 9, 9, 512, 3, 1), (128, 30, 30, 128, 3, 1),
                                                    (64, 56, 56, 128, 1, 2), (64, 58, 58, 64, 3, 1), (128, 28, 28, 256, 1, 2),
-                                                   (256, 16, 16, 512, 3, 2), (64, 58, 58, 128, 3, 2), (128, 30, 30, 256, 3, 2),
-                                                   (256, 14, 14, 512, 1, 2))):
-        a3 = torch.randint(-128, 128, (1, ic // 16, 16, h, w_, 16), dtype=torch.int8, device=dev)
-        w3 = torch.randint(-128, 128, (oc // 16, ic // 16, ks, ks, ks, 4, 16, 4), dtype=torch.int8, device=dev)
+                                                   (256, 16, 16, 512, 3, 2), (64, 58, 58, 128, 3, 2), (4, 230, 230, 64, 7, 2),
+                                                   (128, 30, 30, 256, 3, 2), (256, 14, 14, 512, 1, 2))):
+        cb3 = 4 if ic % 16 else 16   # conv3d.py:39-56
+        a3 = torch.randint(-128, 128, (1, ic // cb3, 16, h, w_, cb3), dtype=torch.int8, device=dev)
+        w3 = torch.randint(-128, 128, (oc // 16, ic // cb3, ks, ks, ks, cb3 // 4, 16, 4), dtype=torch.int8, device=dev)
         od, oh, ow = (16 - ks) // st + 1, (h - ks) // st + 1, (w_ - ks) // st + 1
         o3 = torch.empty((1, oc // 16, od, oh, ow, 16), dtype=torch.int32, device=dev)
         d3 = _lib.Conv3dDesc(1, ic, 16, h, w_, oc, ks, ks, ks, st)
@@ -333,7 +334,8 @@ def main():
         ops = 2.0 * od * oh * ow * oc * ic * ks ** 3
         c3_rows.append(dict(workload=f"{ic}x16x{h}x{w_} -> {oc}, {ks}^3 s{st}", us=round(us, 2),
                             tops=round(ops / us / 1e6, 1), kernel=U.last_variant()))
-    conv3d = dict(workload="3-D int8 convolutions of apps/cpu/kernel/conv3d.py:13-25, NCDHW16c, s8 x s8 -> i32", layers=c3_rows)
+    conv3d = dict(workload="3-D int8 convolutions of apps/cpu/kernel/conv3d.py:13-25, NCDHW16c / NCDHW4c, s8 x s8 -> i32",
+                  layers=c3_rows)
 
     # fp16 variant of the ResNet-50 b32 sweep: valid convolution on pre-padded NCHW16c inputs
     f16_rows, f16_us, f16_flops, f16_ref_us = [], 0.0, 0.0, 0.0

@@ -96,12 +96,13 @@ int unit_conv2d_nchwc_s8s8s32_fused(const unit_conv_desc *d, const void *data, c
  * blocked convolution): valid (no padding), one stride for the three dimensions, s8 x s8 -> i32
  * as its te.compute casts both operands from int8:
  *   O[n,ko,x,y,z,kb] = sum_{ci,rd,rh,rw,e,i} A[n,ci,s*x+rd,s*y+rh,s*z+rw,4e+i] * W[ko,ci,rd,rh,rw,e,kb,i]
- *   data   s8  (N, C/16, D, H, W, 16)
- *   weight s8  (K/16, C/16, KD, KH, KW, 4, 16, 4)
+ *   data   s8  (N, C/cb, D, H, W, cb)
+ *   weight s8  (K/16, C/cb, KD, KH, KW, cb/4, 16, 4)
  *   out    i32 (N, K/16, OD, OH, OW, 16),  O* = (* - K*) / stride + 1
- * 16-channel blocks only (the 4-channel 7x7x7 workload of conv3d.py:22 is not covered). */
+ * The channel block follows conv3d.py:39-56: cb = 16 when C is a multiple of 16, else 4 (C a
+ * multiple of 4; KW <= 8 and KH <= 31 then: its 3 -> 4 channel 7x7x7 workload, conv3d.py:22). */
 typedef struct unit_conv3d_desc {
-  int32_t N, C, D, H, W; /* data: batch, input channels (multiple of 16), depth, height, width */
+  int32_t N, C, D, H, W; /* data: batch, input channels (multiple of 4), depth, height, width */
   int32_t K, KD, KH, KW; /* output channels (multiple of 16), kernel depth, height, width */
   int32_t stride;
 } unit_conv3d_desc;

@@ -72,8 +72,10 @@ def test_out_hw_and_error_paths_without_gpu():
     # the fused signed form and the 3-D operator validate the same way
     assert L.unit_conv2d_nchwc_s8s8s32_fused(ctypes.byref(bad), 1, 1, None, 11, 1, None) == -1
     assert L.unit_conv2d_nchwc_s8s8s32_fused(None, 1, 1, None, 11, 1, None) == -1 and b"null" in L.unit_last_error()
-    d3 = _lib.Conv3dDesc(1, 24, 16, 8, 8, 16, 3, 3, 3, 1)  # C % 16 != 0
-    assert L.unit_conv3d_ncdhwc_s8s8s32(ctypes.byref(d3), 1, 1, 1, None) == -1 and b"multiples of 16" in L.unit_last_error()
+    d3 = _lib.Conv3dDesc(1, 18, 16, 8, 8, 16, 3, 3, 3, 1)  # C % 4 != 0
+    assert L.unit_conv3d_ncdhwc_s8s8s32(ctypes.byref(d3), 1, 1, 1, None) == -1 and b"multiple of 4" in L.unit_last_error()
+    d3 = _lib.Conv3dDesc(1, 4, 16, 20, 20, 16, 3, 3, 9, 1)  # 4-channel blocks: rows of at most 8 taps
+    assert L.unit_conv3d_ncdhwc_s8s8s32(ctypes.byref(d3), 1, 1, 1, None) == -1 and b"KW <= 8" in L.unit_last_error()
     d3 = _lib.Conv3dDesc(1, 16, 2, 8, 8, 16, 3, 3, 3, 1)   # kernel deeper than the input
     assert L.unit_conv3d_ncdhwc_s8s8s32(ctypes.byref(d3), 1, 1, 1, None) == -1 and b"window" in L.unit_last_error()
     assert L.unit_conv_variant_count() >= 70

@@ -225,18 +225,23 @@ CONV3D_CASES = [
     (256, 16, 14, 14, 512, 1, 2),
     (16, 4, 7, 9, 32, 3, 1),      # 27 taps: odd, the last k-step is half padding; ragged pixel count
     (48, 3, 5, 5, 16, (1, 3, 2), 1),
+    (4, 9, 38, 38, 64, 7, 2),     # conv3d.py:22 (230 x 230 there), 3 -> 4 channels: 4-channel blocks
+    (8, 5, 9, 11, 32, (2, 3, 8), 1),   # two 4-channel blocks, rows of 8 taps
+    (12, 4, 6, 7, 48, (3, 1, 5), 2),
 ]
 
 
 @pytest.mark.parametrize("C,D,H,W,K,ks,stride", CONV3D_CASES)
 def test_conv3d_bit_exact(dev, oracle, C, D, H, W, K, ks, stride):
     kd, kh, kw = (ks,) * 3 if isinstance(ks, int) else ks
-    x = rng.uniform_s8((1, C // 16, D, H, W, 16), 17 * C + H)
-    wt = rng.uniform_s8((K // 16, C // 16, kd, kh, kw, 4, 16, 4), 19 * K + kd)
+    cb = 4 if C % 16 else 16     # the channel block rule of apps/cpu/kernel/conv3d.py:39-56
+    x = rng.uniform_s8((1, C // cb, D, H, W, cb), 17 * C + H)
+    wt = rng.uniform_s8((K // 16, C // cb, kd, kh, kw, cb // 4, 16, 4), 19 * K + kd)
     ref = oracle.conv3d_ncdhwc_int8(x, wt, stride)
     out = U.conv3d_NCDHWc_int8(_t(x, dev), _t(wt, dev), stride)
     torch.cuda.synchronize()
     assert tuple(out.shape) == ref.shape
+    assert ("_c4_" in U.last_variant()) == (cb == 4)
     assert np.array_equal(out.cpu().numpy(), ref), U.last_variant()
 
 
@@ -251,6 +256,22 @@ def test_conv3d_every_direct_variant(dev, oracle, monkeypatch):
         out = U.conv3d_NCDHWc_int8(tx, tw, 1)
         torch.cuda.synchronize()
         assert np.array_equal(out.cpu().numpy(), ref), (v, U.last_variant())
+
+
+def test_conv3d_c4_every_direct_variant(dev, oracle, monkeypatch):
+    from unit_amd import _lib
+    x = rng.uniform_s8((2, 2, 6, 8, 13, 4), 31)
+    wt = rng.uniform_s8((3, 2, 3, 2, 5, 1, 16, 4), 37)
+    ref = oracle.conv3d_ncdhwc_int8(x, wt, 1)
+    tx, tw = _t(x, dev), _t(wt, dev)
+    names = set()
+    for v in range(1, _lib.load().unit_conv_variant_count() + 1):
+        monkeypatch.setenv("UNIT_AMD_CONV_VARIANT", str(v))
+        out = U.conv3d_NCDHWc_int8(tx, tw, 1)
+        torch.cuda.synchronize()
+        names.add(U.last_variant())
+        assert np.array_equal(out.cpu().numpy(), ref), (v, U.last_variant())
+    assert len(names) >= 15 and all(n.startswith("s8direct_c4") for n in names), names
 
 
 def test_conv2d_zero_padding_value(dev, oracle):

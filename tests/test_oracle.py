@@ -271,15 +271,18 @@ def test_fused_form_printed_shapes(oracle):
         assert np.array_equal(got.astype(np.int64), want)
 
 
-@pytest.mark.parametrize("c,k,d,hw,ks,stride", [(32, 32, 5, 6, 3, 1), (16, 48, 6, 7, 3, 2), (32, 16, 4, 5, 1, 2)])
+@pytest.mark.parametrize("c,k,d,hw,ks,stride", [(32, 32, 5, 6, 3, 1), (16, 48, 6, 7, 3, 2), (32, 16, 4, 5, 1, 2),
+                                                 (4, 16, 9, 12, 7, 2), (8, 32, 4, 6, 3, 1)])
 def test_conv3d_closed_form(oracle, c, k, d, hw, ks, stride):
     """The restatement of apps/cpu/kernel/conv3d.py:60-64 against torch's float64 conv3d on the
-    un-blocked tensors (an independent library routine; exact at these magnitudes)."""
+    un-blocked tensors (an independent library routine; exact at these magnitudes).  Channel block 16,
+    or 4 when C is not a multiple of 16 (conv3d.py:39-56)."""
+    cb = 4 if c % 16 else 16
     x = oracle.fill_s8((2, c, d, hw, hw), 61)
     w = oracle.fill_s8((k, c, ks, ks, ks), 62)
-    xb = np.ascontiguousarray(x.reshape(2, c // 16, 16, d, hw, hw).transpose(0, 1, 3, 4, 5, 2))
-    # (K, C, kd, kh, kw) -> (K/16, C/16, kd, kh, kw, 4, 16, 4): the conv2d pre-pack with one more window axis
-    wb = np.ascontiguousarray(w.reshape(k // 16, 16, c // 16, 4, 4, ks, ks, ks).transpose(0, 2, 5, 6, 7, 3, 1, 4))
+    xb = np.ascontiguousarray(x.reshape(2, c // cb, cb, d, hw, hw).transpose(0, 1, 3, 4, 5, 2))
+    # (K, C, kd, kh, kw) -> (K/16, C/cb, kd, kh, kw, cb/4, 16, 4): the conv2d pre-pack with one more window axis
+    wb = np.ascontiguousarray(w.reshape(k // 16, 16, c // cb, cb // 4, 4, ks, ks, ks).transpose(0, 2, 5, 6, 7, 3, 1, 4))
     got = oracle.conv3d_ncdhwc_int8(xb, wb, stride)
     want = torch.nn.functional.conv3d(torch.from_numpy(x).double(), torch.from_numpy(w).double(), stride=stride).numpy()
     got_ncdhw = got.transpose(0, 1, 5, 2, 3, 4).reshape(2, k, *got.shape[2:5])

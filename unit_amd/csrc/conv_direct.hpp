@@ -31,12 +31,14 @@
 // that prepare_weight left behind the fragments (passed here as the bias), so the reduction loop
 // does not accumulate weight sums.  The fragment that pads an odd tap count is zero.
 //
-// C4 (with PREP, int8): data in 4-channel blocks (N, C/4, H, W, 4), the layout of the 3-channel
-// stem.  A pixel is 4 bytes, so the KW taps of one window row are consecutive memory: a k-step is
-// one row kh of one channel block, lanes 0-31 hold its taps kw = 0..3 and lanes 32-63 kw = 4..7 (KW <= 8,
-// no dilation along W; prepared weights are zero for kw >= KW).  Each tap is its own dword load with
-// its own mask (row inside the image, per k-step; column inside the image and kw < KW, constant per
-// lane), so no load leaves the tensor.
+// C4 (int8): data in 4-channel blocks (N, C/4, [D,] H, W, 4), the layout of the 3-channel stems.
+// A pixel is 4 bytes, so the KW taps of one window row are consecutive memory: a k-step is one row
+// (ci, kd, kh), lanes 0-31 hold its taps kw = 0..3 and lanes 32-63 kw = 4..7 (KW <= 8, no dilation
+// along W).  Each tap is its own dword load with its own mask (row inside the image, per k-step;
+// column inside the image and kw < KW, constant per lane), so no load leaves the tensor.  Taps
+// kw >= KW carry masked data; their weights are zeros in prepared form, and with the reference's
+// layout (K/16, C/4, [KD,] KH, KW, 1, 16, 4) they re-read tap KW - 1, which is harmless for the same
+// reason as the odd tap above: masked data times any weight cancels (u8) or is zero (s8).
 #pragma once
 #include "epilogues.hpp"
 #include "loaders.hpp"
@@ -118,7 +120,7 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
   constexpr int TAPB = C4 ? 4 : (kInt ? 16 : 32);  // bytes of one pixel and tap
   constexpr int WTAP = kInt ? 256 : 512;           // bytes of one tap of a 16-channel weight block
   static_assert(kInt || (!SHIFT && !S::PAD), "the fp16 operator has neither a shift nor padding");
-  static_assert(!C4 || (kInt && PREP && S::PAD), "4-channel blocks: int8 on prepared weights, masked loads");
+  static_assert(!C4 || (kInt && S::PAD), "4-channel blocks: int8, masked loads");
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int l32 = lane & 31, half = lane >> 5;
@@ -139,9 +141,10 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
   for (int e = threadIdx.x; e < ntab; e += S::NT) {
     v2i ent = {0, 31};
     if constexpr (C4) {
-      int ci, kh;
-      g.by_kh.divmod(e >> 1, ci, kh);
-      ent[0] = ((ci * g.H + kh * g.dh) * g.W) * 4 + (e & 1) * 16;
+      int rest, kh, ci, kd;
+      g.by_kh.divmod(e >> 1, rest, kh);
+      g.by_kd.divmod(rest, ci, kd);
+      ent[0] = (((ci * g.D + kd) * g.H + kh * g.dh) * g.W) * 4 + (e & 1) * 16;
       ent[1] = g.nopad ? 0 : kh;
     } else if (e < g.ntaps) {
       int kw, rest, kh, rest2, kd, ci;
@@ -173,7 +176,15 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
     if constexpr (PREP) {  // blocks past the last one re-read it
       const int kb = min((x0 >> 5) + i, (ep.K - 1) >> 5);
       xoff[i] = ((u32)(kb * nsteps) * 64u + (u32)lane) * 16u;
+    } else if constexpr (C4) {  // a tap of a 16-channel block is 64 bytes, a window row KW of them
+      xoff[i] = (u32)(n >> 4) * (u32)(g.ntaps * 64) + (u32)(n & 15) * 4u;
     }
+  }
+  // C4 on the reference's weight layout: byte offset of this lane's four taps inside a window row
+  u32 wtap[C4 && !PREP ? 4 : 1];
+  if constexpr (C4 && !PREP) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) wtap[e] = (u32)min(4 * half + e, g.KW - 1) * 64u;
   }
   // per-channel addend read from memory (bias; with PREP and u8 data the shift correction): one
   // wave contributes it, and the load is issued here so that its latency hides behind the loop
@@ -250,7 +261,8 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
   auto fetch = [&](auto slot) __attribute__((always_inline)) {
     constexpr int U = decltype(slot)::value;
     const int t = kInt ? 2 * sf + half : sf;
-    const u32 xs = (u32)sf * 1024u;  // PREP: a k-step of a 32-channel block is 1 KiB
+    const int scur = sf;
+    const u32 xs = (u32)scur * 1024u;  // PREP: a k-step of a 32-channel block is 1 KiB
     const v2i e = ecur;
     sf = sf < slast ? sf + 1 : slast;
     ecur = tab[kInt ? 2 * sf + half : sf];
@@ -264,6 +276,10 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
       const u32 o = xoff[i] + xk;
       if constexpr (PREP) {
         xf[U][i] = *reinterpret_cast<const v4i *>(wgt + xoff[i] + xs);
+      } else if constexpr (C4) {
+        const u32 xr = (u32)scur * (u32)(g.KW * 64);  // this k-step's window row
+#pragma unroll
+        for (int d = 0; d < 4; ++d) xf[U][i][d] = *reinterpret_cast<const int *>(wgt + xoff[i] + xr + wtap[d]);
       } else if constexpr (kInt) {
 #pragma unroll
         for (int d = 0; d < 4; ++d) xf[U][i][d] = *reinterpret_cast<const int *>(wgt + o + d * 64);

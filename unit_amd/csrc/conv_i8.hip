@@ -8,6 +8,9 @@ int conv_i8_c16(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g
                 void *out, hipStream_t s);
 int conv_i8_direct(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
                    void *out, hipStream_t s);
+bool conv_c4_direct_ok(const unit_conv_desc *d);  // conv_direct_c4.hip
+int conv_c4_direct(const char *what, const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data,
+                   const void *w, const int *bias, int scale, bool shift, void *out, hipStream_t s);
 int conv_i8_c4(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
                void *out, hipStream_t s);
 
@@ -46,7 +49,12 @@ extern "C" int unit_conv2d_nchwc_u8s8s32(const unit_conv_desc *d, const void *da
   if (int rc = check_device()) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int ntable = (int)(sizeof(kTunedI8) / sizeof(kTunedI8[0])) - 1;
-  const ConvPlan p = plan_conv(d, g.npix, g.ntaps * d->cb, kTunedI8, ntable, true, d->cb == 16 && d->KH * d->KW <= 31);
-  if (kConvTiles[p.variant].direct) return conv_i8_direct(p, d, g, data, weight, out, s);
+  const bool direct_ok = d->cb == 16 ? d->KH * d->KW <= 31 : conv_c4_direct_ok(d);
+  const ConvPlan p = plan_conv(d, g.npix, g.ntaps * d->cb, kTunedI8, ntable, true, direct_ok);
+  if (kConvTiles[p.variant].direct) {
+    if (!direct_ok) return fail(UNIT_E_ARG, "%s: kernel variant %d not available for this layout or window", what, p.variant);
+    return d->cb == 16 ? conv_i8_direct(p, d, g, data, weight, out, s)
+                       : conv_c4_direct(what, p, d, g, data, weight, nullptr, 1, true, out, s);
+  }
   return d->cb == 16 ? conv_i8_c16(p, d, g, data, weight, out, s) : conv_i8_c4(p, d, g, data, weight, out, s);
 }

@@ -1,8 +1,8 @@
 // C-ABI entry and kernels of the fused signed int8 convolution
 //   out = (sum x_s8 * w + bias[k]) * scale
 // = the reference's fused_nn_contrib_conv2d_NCHWc_subtract_add_multiply on x + 128
-// (apps/cpu/relay/result.log:3-26,35).  NCHW16c with windows of up to 31 positions runs on the
-// direct kernels; everything else (NCHW4c stems, larger windows) on two staged tile shapes.
+// (apps/cpu/relay/result.log:3-26,35).  NCHW16c with windows of up to 31 positions and NCHW4c with
+// rows of up to 8 taps run on the direct kernels; everything else on two staged tile shapes.
 #include "conv_direct_host.hpp"
 #include "conv_i8_impl.hpp"
 
@@ -10,6 +10,9 @@ namespace unit {
 
 int conv_geom(const unit_conv_desc *d, int tapb, ConvGeom *g, const char *what);  // abi.hip
 const TunedConv *tuned_conv_i8(int *n);                                             // conv_i8.hip
+bool conv_c4_direct_ok(const unit_conv_desc *d);                                    // conv_direct_c4.hip
+int conv_c4_direct(const char *what, const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data,
+                   const void *w, const int *bias, int scale, bool shift, void *out, hipStream_t s);
 
 // direct kernels on signed data; `what` names the entry point in messages (also used by the 3-D operator)
 int conv_s8_direct(const char *kWhat, const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data,
@@ -60,13 +63,14 @@ extern "C" int unit_conv2d_nchwc_s8s8s32_fused(const unit_conv_desc *d, const vo
   if (int rc = check_aligned(kWhat, {data, weight, out})) return rc;
   if (int rc = check_device()) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (d->cb == 16 && d->KH * d->KW <= 31) {
+  if (d->cb == 16 ? d->KH * d->KW <= 31 : conv_c4_direct_ok(d)) {
     // same shapes, same kernels as the unsigned operator minus shift and weight sums: its plan serves
     int ntable = 0;
     const TunedConv *table = tuned_conv_i8(&ntable);
-    ConvPlan p = plan_conv(d, g.npix, g.ntaps * 16, table, ntable, true, true);
-    if (!kConvTiles[p.variant].direct) p = heuristic_plan(g.npix, d->K, g.ntaps * 16, true, true);
+    ConvPlan p = plan_conv(d, g.npix, g.ntaps * d->cb, table, ntable, true, true);
+    if (!kConvTiles[p.variant].direct) p = heuristic_plan(g.npix, d->K, g.ntaps * d->cb, true, true);
     p.splits = 1;
+    if (d->cb == 4) return conv_c4_direct(kWhat, p, d, g, data, weight, bias, scale, false, out, s);
     return conv_s8_direct(kWhat, p, d, g, data, weight, bias, scale, out, s);
   }
   return d->cb == 16 ? staged_s8<16>(d, g, data, weight, bias, scale, out, s)

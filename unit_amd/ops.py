@@ -253,8 +253,8 @@ def conv3d_NCDHWc_int8(data, kernel, stride=1):
     """The 3-D blocked convolution of apps/cpu/kernel/conv3d.py:39-64: valid, one stride for depth,
     height and width, int8 x int8 -> int32 (its te.compute casts both placeholders from int8).
 
-    data   int8  (N, C/16, D, H, W, 16)
-    kernel int8  (K/16, C/16, KD, KH, KW, 4, 16, 4)
+    data   int8  (N, C/cb, D, H, W, cb), cb = 16, or 4 with KW <= 8 (the file's 3 -> 4 channel workload)
+    kernel int8  (K/16, C/cb, KD, KH, KW, cb/4, 16, 4)
     returns int32 (N, K/16, OD, OH, OW, 16)
     """
     import ctypes
@@ -262,15 +262,15 @@ def conv3d_NCDHWc_int8(data, kernel, stride=1):
     kernel = _dev(kernel, "kernel", torch.int8, 8)
     n, cc, dd, h, w, cb = data.shape
     ko, cc2, kd, kh, kw, e, kb, i4 = kernel.shape
-    if cb != 16:
-        raise ValueError(f"data: the 3-D operator takes 16-channel blocks, got {cb}")
-    if (cc2, e, kb, i4) != (cc, 4, 16, 4):
+    if cb not in (4, 16) or (cb == 4 and (cc * cb) % 16 == 0):
+        raise ValueError(f"data: channel block must be 16, or 4 when C is not a multiple of 16 (got {cb}, C = {cc * cb})")
+    if (cc2, e, kb, i4) != (cc, cb // 4, 16, 4):
         raise ValueError(f"kernel: shape {tuple(kernel.shape)} does not match data {tuple(data.shape)}; "
-                         f"expected (K/16, {cc}, KD, KH, KW, 4, 16, 4)")
+                         f"expected (K/16, {cc}, KD, KH, KW, {cb // 4}, 16, 4)")
     stride = int(stride)
     if stride <= 0 or kd > dd or kh > h or kw > w:
         raise ValueError("stride must be positive and the kernel window must fit the input")
-    d = _lib.Conv3dDesc(n, cc * 16, dd, h, w, ko * 16, kd, kh, kw, stride)
+    d = _lib.Conv3dDesc(n, cc * cb, dd, h, w, ko * 16, kd, kh, kw, stride)
     od, oh, ow = (dd - kd) // stride + 1, (h - kh) // stride + 1, (w - kw) // stride + 1
     out = torch.empty((n, ko, od, oh, ow, 16), dtype=torch.int32, device=data.device)
     check(_lib.load().unit_conv3d_ncdhwc_s8s8s32(ctypes.byref(d), data.data_ptr(), kernel.data_ptr(), out.data_ptr(),
