@@ -7,16 +7,18 @@
 namespace unit {
 namespace {
 
-template <class T, bool OUT_F16, int PF = 1>
+// TAIL = false: K is a whole number of stages (the loaders then stage without zeroing selects)
+template <class T, bool OUT_F16, int PF = 1, bool TAIL = true>
 int run_gemm_f16(const void *a, const void *b, void *c, int M, int N, int K, hipStream_t s) {
-  using XL = RowMajorLoader<T::BX, T::BKB, T::NT, false, PF>;
-  using YL = KMajorF16Loader<T::BY, T::BKB, T::NT, PF>;
+  using XL = RowMajorLoader<T::BX, T::BKB, T::NT, false, PF, TAIL>;
+  using YL = KMajorF16Loader<T::BY, T::BKB, T::NT, PF, TAIL>;
   using Epi = GemmEpilogue<OpF16, OUT_F16>;
   typename XL::Params xp{static_cast<const char *>(a), M, K * 2, K * 2};
   typename YL::Params yp{static_cast<const char *>(b), N, K, N + 4, 0, N * 2};
   typename Epi::Params ep{c, M, N};
   const int nk = ceil_div(K * 2, T::BKB), gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
-  set_variant("f16gemm_x%d_y%d_k%d_w%dx%d_p%d%s", T::BX, T::BY, T::BKB, T::WX, T::WY, PF, OUT_F16 ? "_h" : "");
+  set_variant("f16gemm_x%d_y%d_k%d_w%dx%d_p%d%s%s", T::BX, T::BY, T::BKB, T::WX, T::WY, PF, TAIL ? "" : "e",
+              OUT_F16 ? "_h" : "");
   return launch_mma<OpF16, T, XL, YL, Epi, WS_NONE>(xp, yp, ep, nk, gx, gy, 4, 1, c, 0, 0, s, "unit_gemm_f16");
 }
 
@@ -34,7 +36,9 @@ int gemm_f16(const void *a, const void *b, void *c, int M, int N, int K, hipStre
     default: break;
   }
   // 64 (m) x 128 (n) wave tiles: measured 8-10 % faster than 128 x 64 (512-byte row runs per wave in the write-back)
-  if (M >= 256 && N >= 256 && tiles_big >= 128) return run_gemm_f16<Tile<256, 256, 128, 4, 2>, OUT_F16>(a, b, c, M, N, K, s);
+  if (M >= 256 && N >= 256 && tiles_big >= 128)
+    return K % 64 ? run_gemm_f16<Tile<256, 256, 128, 4, 2>, OUT_F16>(a, b, c, M, N, K, s)
+                  : run_gemm_f16<Tile<256, 256, 128, 4, 2>, OUT_F16, 1, false>(a, b, c, M, N, K, s);
   return run_gemm_f16<Tile<128, 128, 64, 2, 2>, OUT_F16>(a, b, c, M, N, K, s);
 }
 

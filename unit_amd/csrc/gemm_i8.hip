@@ -9,11 +9,12 @@
 namespace unit {
 namespace {
 
-template <class T, bool PACKED>
+// TAIL = false: K is a whole number of stages (the loaders then stage without zeroing selects)
+template <class T, bool PACKED, bool TAIL = true>
 int run_dense(const void *a, const void *w, void *c, int M, int N, int K, hipStream_t s) {
-  using XL = RowMajorLoader<T::BX, T::BKB, T::NT, true>;
-  using YLrm = RowMajorLoader<T::BY, T::BKB, T::NT, false>;
-  using YLpk = VnniLoader<T::BY, T::BKB, T::NT, 128>;
+  using XL = RowMajorLoader<T::BX, T::BKB, T::NT, true, 1, TAIL>;
+  using YLrm = RowMajorLoader<T::BY, T::BKB, T::NT, false, 1, TAIL>;
+  using YLpk = VnniLoader<T::BY, T::BKB, T::NT, 128, 1, TAIL>;
   using Epi = GemmEpilogue<OpI8, false>;
   typename XL::Params xp{static_cast<const char *>(a), M, K, K};
   typename Epi::Params ep{c, M, N};
@@ -25,7 +26,8 @@ int run_dense(const void *a, const void *w, void *c, int M, int N, int K, hipStr
   }
   if (splits > nk) splits = nk;
   if ((size_t)M * N * 4 % 16) splits = 1;
-  set_variant("i8dense%s_x%d_y%d_k%d_w%d_s%d", PACKED ? "pk" : "rm", T::BX, T::BY, T::BKB, T::NT / 64, splits);
+  set_variant("i8dense%s_x%d_y%d_k%d_w%d%s_s%d", PACKED ? "pk" : "rm", T::BX, T::BY, T::BKB, T::NT / 64, TAIL ? "" : "e",
+              splits);
   if constexpr (PACKED) {
     typename YLpk::Params yp{static_cast<const char *>(w), N, K / 4};
     return launch_mma<OpI8, T, XL, YLpk, Epi, WS_Y>(xp, yp, ep, nk, gx, gy, 4, splits, c, (size_t)M * N * 4, 0, s,
@@ -120,7 +122,9 @@ int dense(const void *a, const void *w, void *c, int M, int N, int K, unit_strea
     case 15: return run_dense<Tile<256, 256, 128, 4, 2>, PACKED>(a, w, c, M, N, K, s);
     default: break;
   }
-  if (M >= 256 && N >= 256 && tiles_big >= 128) return run_dense<Tile<256, 256, 128, 2, 4>, PACKED>(a, w, c, M, N, K, s);
+  if (M >= 256 && N >= 256 && tiles_big >= 128)
+    return K % 128 ? run_dense<Tile<256, 256, 128, 2, 4>, PACKED>(a, w, c, M, N, K, s)
+                   : run_dense<Tile<256, 256, 128, 2, 4>, PACKED, false>(a, w, c, M, N, K, s);
   return run_dense<Tile<128, 128, 64, 2, 2>, PACKED>(a, w, c, M, N, K, s);
 }
 

@@ -11,8 +11,11 @@ __device__ __forceinline__ v4i zero4() { return v4i{0, 0, 0, 0}; }
 // Rows that are K-contiguous in memory: GEMM A (M, K) u8 / f16 and W (N, K) s8.
 // Thread t owns chunk column t % CPR of rows t / CPR + i * NT / CPR: 8 (or 4) consecutive lanes
 // read one whole 128-byte (64-byte) row segment.
+// TAIL = false (all three k-contiguous loaders): the reduction is a whole number of stages, so no
+// chunk lies past its end and the select instructions that zero such chunks (one per staged
+// dword) are left out.
 // ------------------------------------------------------------------------------------------
-template <int ROWS, int BKB, int NT, bool XOR80, int PF = 1>
+template <int ROWS, int BKB, int NT, bool XOR80, int PF = 1, bool TAIL = true>
 struct RowMajorLoader {
   struct Params {
     const char *base;
@@ -50,7 +53,7 @@ struct RowMajorLoader {
   __device__ __forceinline__ void fetch(int kt) {
     // loads are unconditional (no branches in the pipeline): a chunk past the end of the
     // reduction re-reads the first chunk of the row and is zeroed when it is written to LDS
-    const bool ok = kt * BKB < kleft;
+    const bool ok = !TAIL || kt * BKB < kleft;
     const int kb = ok ? kt * BKB + coff : 0;
     okm[S] = ok;
 #pragma unroll
@@ -60,7 +63,7 @@ struct RowMajorLoader {
   __device__ __forceinline__ void commit(char *tile) {
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      v4i v = okm[S] ? r[S][i] : zero4();
+      v4i v = (!TAIL || okm[S]) ? r[S][i] : zero4();
       if (XOR80) v ^= (int)0x80808080;
       *reinterpret_cast<v4i *>(tile + ldsoff + i * RPP * BKB) = v;
     }
@@ -74,7 +77,7 @@ struct RowMajorLoader {
 // A thread loads, for 4 consecutive n, the 4 k-groups of one 16-byte reduction chunk (4 x 16
 // bytes), transposes the 4x4 dwords in registers (free) and writes one 16-byte LDS chunk per n.
 // ------------------------------------------------------------------------------------------
-template <int ROWS, int BKB, int NT, int NB, int PF = 1>
+template <int ROWS, int BKB, int NT, int NB, int PF = 1, bool TAIL = true>
 struct VnniLoader {
   struct Params {
     const char *base;
@@ -121,7 +124,7 @@ struct VnniLoader {
 #pragma unroll
       for (int d = 0; d < 4; ++d) {
         // unconditional load: a k-group past the end re-reads k-group 0
-        const int kg = kg0 + d < kg_total ? kg0 + d : 0;
+        const int kg = (!TAIL || kg0 + d < kg_total) ? kg0 + d : 0;
         r[S][i][d] = *reinterpret_cast<const v4i *>(ptr[i] + (size_t)kg * kgstride);
       }
     }
@@ -131,7 +134,7 @@ struct VnniLoader {
     if (!active) return;
 #pragma unroll
     for (int i = 0; i < UPT; ++i) {
-      const int left = kg_total - (kt_of[S] * CPR + cidx[i]) * 4;  // valid k-groups of this chunk
+      const int left = TAIL ? kg_total - (kt_of[S] * CPR + cidx[i]) * 4 : 4;  // valid k-groups of this chunk
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         v4i v = {left > 0 ? r[S][i][0][j] : 0, left > 1 ? r[S][i][1][j] : 0, left > 2 ? r[S][i][2][j] : 0,
@@ -148,7 +151,7 @@ struct VnniLoader {
 // + (n % NBLK) * 2.  A thread loads an 8 (k) x 4 (n) patch as 8 x 8 bytes, transposes it with
 // v_perm_b32 and writes one 16-byte chunk (8 k) per n.
 // ------------------------------------------------------------------------------------------
-template <int ROWS, int BKB, int NT, int PF = 1>
+template <int ROWS, int BKB, int NT, int PF = 1, bool TAIL = true>
 struct KMajorF16Loader {
   struct Params {
     const char *base;
@@ -192,7 +195,7 @@ struct KMajorF16Loader {
 #pragma unroll
     for (int i = 0; i < UPT; ++i) {
       const int k0 = (kt * CPR + cidx[i]) * 8;
-      const bool ok = k0 < ktotal;  // ktotal % 8 == 0: a chunk is all valid or all padding
+      const bool ok = !TAIL || k0 < ktotal;  // ktotal % 8 == 0: a chunk is all valid or all padding
       // unconditional loads: a chunk past the end re-reads rows 0..7
       const char *q = ptr[i] + (ok ? (size_t)k0 * row_stride : 0);
       okm[S][i] = ok;
@@ -212,7 +215,7 @@ struct KMajorF16Loader {
         v4i v;
 #pragma unroll
         for (int p = 0; p < 4; ++p)
-          v[p] = okm[S][i] ? (int)__builtin_amdgcn_perm((u32)r[S][i][2 * p + 1][j >> 1], (u32)r[S][i][2 * p][j >> 1], sel) : 0;
+          v[p] = (!TAIL || okm[S][i]) ? (int)__builtin_amdgcn_perm((u32)r[S][i][2 * p + 1][j >> 1], (u32)r[S][i][2 * p][j >> 1], sel) : 0;
         *reinterpret_cast<v4i *>(tile + lds_off<BKB>(lrow[i] + j, cidx[i])) = v;
       }
   }
