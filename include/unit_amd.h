@@ -174,6 +174,17 @@ int unit_prepack_dense_weight_s8(const void *src, void *dst, int32_t N, int32_t 
 int unit_prepack_conv_weight_f16(const void *src, void *dst, int32_t O, int32_t I, int32_t KH,
                                  int32_t KW, unit_stream_t stream);
 
+/* The same GEMM with b prepared once: bt f16 (N, K) = b^T, K-contiguous like a, so that both
+ * operand tiles go from global memory straight into LDS (no register round trip, no transposition
+ * while staging).  The reference's analogue is the one-time re-layout of b in
+ * apps/gpu/gemm-pack.py:9,17 (b pre-packed as (N/32, K/32, 32, 32) for its wmma loads).
+ * unit_gemm_f16_prepare_b writes bt (N * K halves, caller-owned) from b (K, N); K % 8 == 0.
+ * unit_gemm_f16_prepared: c (M, N) = a (M, K) . bt^T, same results as unit_gemm_f16 (the same
+ * products summed in the same order); K % 8 == 0, N % 4 == 0. */
+int unit_gemm_f16_prepare_b(const void *b, void *bt, int32_t K, int32_t N, unit_stream_t stream);
+int unit_gemm_f16_prepared(const void *a, const void *bt, void *c, int32_t M, int32_t N, int32_t K,
+                           int32_t out_f16, unit_stream_t stream);
+
 /* Alignment: every tensor pointer passed to a convolution, dense, GEMM or prepare entry point
  * must be 16-byte aligned (the kernels use 16-byte vector accesses); a misaligned one is
  * rejected with UNIT_E_ARG.  Framework allocations (256 bytes and up) satisfy this; a view that

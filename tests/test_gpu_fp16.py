@@ -49,6 +49,41 @@ def test_gemm_fp16(dev, oracle, M, N, K, out_dtype):
     assert err <= (REL_TOL if out_dtype == "float32" else REL_TOL), (err, U.last_variant())
 
 
+PREPARED_GEMM_CASES = GEMM_CASES + [(4096, 4096, 1024), (2304, 2560, 192), (257, 260, 64), (3000, 2052, 200)]
+
+
+@pytest.mark.parametrize("M,N,K", PREPARED_GEMM_CASES)
+@pytest.mark.parametrize("out_dtype", ["float32", "float16"])
+def test_gemm_fp16_prepared_b(dev, oracle, M, N, K, out_dtype):
+    """b re-laid once as (N, K): the transposed buffer is exact, the product is within tolerance of float64 and
+    agrees with the plain entry to rounding (both sum k in ascending order of 16-element MFMA steps)."""
+    a = rng.normal_f16((M, K), 31 + M, 1.0 / np.sqrt(K))
+    b = rng.normal_f16((K, N), 57 + N)
+    ta, tb = _t(a, dev), _t(b, dev)
+    pb = U.prepare_gemm_b(tb)
+    torch.cuda.synchronize()
+    assert np.array_equal(pb.bt.cpu().numpy(), b.T)
+    out = U.gemm_fp16(ta, pb, out_dtype)
+    torch.cuda.synchronize()
+    assert U.last_variant().startswith("f16gemmbt")
+    ref = oracle.gemm_f16(a, b)
+    err = max_rel(out.cpu().numpy(), ref)
+    assert err <= REL_TOL, (err, U.last_variant())
+    plain = U.gemm_fp16(ta, tb, out_dtype)
+    assert max_rel(out.cpu().numpy(), plain.cpu().numpy().astype(np.float64)) <= 1e-3, U.last_variant()
+
+
+def test_gemm_fp16_prepared_b_integer_exact(dev, oracle):
+    M, N, K = 512, 768, 1024   # large enough for the direct-to-LDS kernel (256 x 256 tiles, K % 64 == 0)
+    a = (np.arange(M * K).reshape(M, K) % 7).astype(np.float16)
+    b = (np.arange(K * N).reshape(K, N) % 5 - 2).astype(np.float16)
+    for m, n in ((M, N), (4096, 2048)):
+        aa = np.resize(a, (m, K)); bb = np.resize(b, (K, n))
+        out = U.gemm_fp16(_t(aa, dev), U.prepare_gemm_b(_t(bb, dev))).cpu().numpy()
+        assert np.array_equal(out.astype(np.float64), oracle.gemm_f16(aa, bb)), U.last_variant()
+    assert "dma" in U.last_variant()
+
+
 def test_gemm_fp16_integer_exact(dev, oracle):
     """Small-integer operands (the arange % 7 recipe of apps/gpu/conv-wdim.py:33-36) make every
     fp32 partial sum exact, so the result must match the float64 reference bit for bit."""

@@ -3,9 +3,72 @@
 #include "epilogues.hpp"
 #include "host.hpp"
 #include "loaders.hpp"
+#include "mma_dma.hpp"
 
 namespace unit {
 namespace {
+
+// Prepared b: (N, K) rows, K-contiguous like a.  Both operands then go global -> LDS directly
+// (no register round trip, no transposition), through a ring of NSTAGE LDS buffers; K a whole
+// number of stages.
+template <class T, int NSTAGE, bool OUT_F16>
+int run_gemm_f16_bt_dma(const void *a, const void *bt, void *c, int M, int N, int K, hipStream_t s) {
+  using Epi = GemmEpilogue<OpF16, OUT_F16>;
+  DmaParams p{static_cast<const char *>(a), static_cast<const char *>(bt), M, N, K * 2};
+  typename Epi::Params ep{c, M, N};
+  const int nk = K * 2 / T::BKB, gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
+  constexpr int lds = NSTAGE * T::STAGE;
+  static_assert(lds <= kMaxLds, "ring does not fit the LDS");
+  auto kern = mma_dma_kernel<OpF16, T, NSTAGE, Epi, WS_NONE, false>;
+  static thread_local bool allowed = false;
+  if (!allowed) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
+    if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "unit_gemm_f16_prepared: hipFuncSetAttribute: %s", hipGetErrorString(e));
+    allowed = true;
+  }
+  GridMap gm{gx, gy, gx < 4 ? gx : 4, 1, gx * gy};
+  set_variant("f16gemmbt_dma_x%d_y%d_k%d_w%dx%d_r%d%s", T::BX, T::BY, T::BKB, T::WX, T::WY, NSTAGE, OUT_F16 ? "_h" : "");
+  hipLaunchKernelGGL(kern, dim3(gm.total), dim3(T::NT), lds, s, p, ep, nk, gm);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "unit_gemm_f16_prepared: launch: %s", hipGetErrorString(e));
+}
+
+// the same operands through registers (any K that is a multiple of 8; small problems)
+template <class T, bool OUT_F16>
+int run_gemm_f16_bt(const void *a, const void *bt, void *c, int M, int N, int K, hipStream_t s) {
+  using XL = RowMajorLoader<T::BX, T::BKB, T::NT, false>;
+  using YL = RowMajorLoader<T::BY, T::BKB, T::NT, false>;
+  using Epi = GemmEpilogue<OpF16, OUT_F16>;
+  typename XL::Params xp{static_cast<const char *>(a), M, K * 2, K * 2};
+  typename YL::Params yp{static_cast<const char *>(bt), N, K * 2, K * 2};
+  typename Epi::Params ep{c, M, N};
+  const int nk = ceil_div(K * 2, T::BKB), gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
+  set_variant("f16gemmbt_x%d_y%d_k%d_w%dx%d%s", T::BX, T::BY, T::BKB, T::WX, T::WY, OUT_F16 ? "_h" : "");
+  return launch_mma<OpF16, T, XL, YL, Epi, WS_NONE>(xp, yp, ep, nk, gx, gy, 4, 1, c, 0, 0, s, "unit_gemm_f16_prepared");
+}
+
+template <bool OUT_F16>
+int gemm_f16_bt(const void *a, const void *bt, void *c, int M, int N, int K, hipStream_t s) {
+  const long tiles_big = (long)ceil_div(M, 256) * ceil_div(N, 256);
+  if (M >= 256 && N >= 256 && tiles_big >= 128) {
+    if (K % 64 == 0 && K >= 128) return run_gemm_f16_bt_dma<Tile<256, 256, 128, 2, 4>, 2, OUT_F16>(a, bt, c, M, N, K, s);
+    return run_gemm_f16_bt<Tile<256, 256, 128, 2, 4>, OUT_F16>(a, bt, c, M, N, K, s);
+  }
+  return run_gemm_f16_bt<Tile<128, 128, 64, 2, 2>, OUT_F16>(a, bt, c, M, N, K, s);
+}
+
+// b (K, N) -> bt (N, K): 64 x 64 tiles through LDS, 128-byte row segments on both sides
+__global__ __launch_bounds__(256) void transpose_f16(const _Float16 *__restrict__ b, _Float16 *__restrict__ bt, int K,
+                                                     int N) {
+  __shared__ _Float16 tile[64][66];
+  const int k0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int r = ty; r < 64; r += 4)
+    if (k0 + r < K && n0 + tx < N) tile[r][tx] = b[(size_t)(k0 + r) * N + n0 + tx];
+  __syncthreads();
+  for (int r = ty; r < 64; r += 4)
+    if (n0 + r < N && k0 + tx < K) bt[(size_t)(n0 + r) * K + k0 + tx] = tile[tx][r];
+}
 
 // TAIL = false: K is a whole number of stages (the loaders then stage without zeroing selects)
 template <class T, bool OUT_F16, int PF = 1, bool TAIL = true>
@@ -59,4 +122,37 @@ extern "C" int unit_gemm_f16(const void *a, const void *b, void *c, int32_t M, i
   if (int rc = check_device()) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   return out_f16 ? gemm_f16<true>(a, b, c, M, N, K, s) : gemm_f16<false>(a, b, c, M, N, K, s);
+}
+
+extern "C" int unit_gemm_f16_prepare_b(const void *b, void *bt, int32_t K, int32_t N, unit_stream_t stream) {
+  using namespace unit;
+  const char *what = "unit_gemm_f16_prepare_b";
+  if (!b || !bt) return fail(UNIT_E_ARG, "%s: null pointer", what);
+  if (K <= 0 || N <= 0) return fail(UNIT_E_ARG, "%s: K, N must be positive (got %d, %d)", what, K, N);
+  if (K % 8) return fail(UNIT_E_ARG, "%s: K must be a multiple of 8 (got %d)", what, K);
+  if (!fits((size_t)N * K * 2)) return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
+  if (int rc = check_aligned(what, {b, bt})) return rc;
+  if (int rc = check_device()) return rc;
+  hipLaunchKernelGGL(transpose_f16, dim3(ceil_div(N, 64), ceil_div(K, 64)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const _Float16 *>(b), static_cast<_Float16 *>(bt), K, N);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "%s: launch: %s", what, hipGetErrorString(e));
+  set_variant("f16_transpose_b");
+  return UNIT_OK;
+}
+
+extern "C" int unit_gemm_f16_prepared(const void *a, const void *bt, void *c, int32_t M, int32_t N, int32_t K,
+                                      int32_t out_f16, unit_stream_t stream) {
+  using namespace unit;
+  const char *what = "unit_gemm_f16_prepared";
+  if (!a || !bt || !c) return fail(UNIT_E_ARG, "%s: null pointer", what);
+  if (M <= 0 || N <= 0 || K <= 0) return fail(UNIT_E_ARG, "%s: M, N, K must be positive (got %d, %d, %d)", what, M, N, K);
+  if (K % 8) return fail(UNIT_E_ARG, "%s: K must be a multiple of 8 (got %d)", what, K);
+  if (N % 4) return fail(UNIT_E_ARG, "%s: N must be a multiple of 4 (got %d)", what, N);
+  if (!fits((size_t)M * K * 2) || !fits((size_t)N * K * 2) || !fits((size_t)M * N * 4))
+    return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
+  if (int rc = check_aligned(what, {a, bt, c})) return rc;
+  if (int rc = check_device()) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return out_f16 ? gemm_f16_bt<true>(a, bt, c, M, N, K, s) : gemm_f16_bt<false>(a, bt, c, M, N, K, s);
 }

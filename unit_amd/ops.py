@@ -21,7 +21,7 @@ __all__ = [
     "conv2d_NCHWc_int8", "dense_dotprod", "dense", "conv2d_NCHW16c_OHWI16o", "gemm_fp16",
     "pack_nchwc", "unpack_nchwc", "prepack_conv_weight", "prepack_dense_weight",
     "prepack_conv_weight_f16", "conv_out_hw", "last_variant",
-    "PreparedConvWeight", "prepare_conv2d_weight",
+    "PreparedConvWeight", "prepare_conv2d_weight", "PreparedGemmB", "prepare_gemm_b",
 ]
 
 
@@ -312,17 +312,45 @@ def dense(data, weight, out_dtype="int32"):
 
 
 # ------------------------------------------------------------------------------- fp16
-def gemm_fp16(a, b, out_dtype="float32"):
-    """c[x, y] = sum_k f32(a[x, k]) * f32(b[k, y]); a (M, K), b (K, N) fp16 row-major."""
-    a = _dev(a, "a", torch.float16, 2)
+class PreparedGemmB:
+    """The b operand of gemm_fp16 re-laid once as (N, K) (see prepare_gemm_b)."""
+
+    def __init__(self, bt, K, N):
+        self.bt, self.K, self.N = bt, K, N
+
+    def __repr__(self):
+        return f"PreparedGemmB(K={self.K}, N={self.N})"
+
+
+def prepare_gemm_b(b):
+    """Re-lay the constant operand b (K, N) of gemm_fp16 once as (N, K), the counterpart of the one-time
+    packing of b in apps/gpu/gemm-pack.py:9,17; gemm_fp16 accepts the result in place of b."""
     b = _dev(b, "b", torch.float16, 2)
+    k, n = b.shape
+    bt = torch.empty((n, k), dtype=torch.float16, device=b.device)
+    check(_lib.load().unit_gemm_f16_prepare_b(b.data_ptr(), bt.data_ptr(), k, n, _stream()))
+    return PreparedGemmB(bt, k, n)
+
+
+def gemm_fp16(a, b, out_dtype="float32"):
+    """c[x, y] = sum_k f32(a[x, k]) * f32(b[k, y]); a (M, K), b (K, N) fp16 row-major, or b a
+    PreparedGemmB."""
+    a = _dev(a, "a", torch.float16, 2)
     if out_dtype not in ("float32", "float16"):
         raise ValueError(f"out_dtype: expected 'float32' or 'float16', got {out_dtype!r}")
     m, k = a.shape
+    half = out_dtype == "float16"
+    if isinstance(b, PreparedGemmB):
+        if b.K != k or b.bt.device != a.device:
+            raise ValueError(f"b: {b!r} does not match a {tuple(a.shape)} on {a.device}")
+        out = torch.empty((m, b.N), dtype=torch.float16 if half else torch.float32, device=a.device)
+        check(_lib.load().unit_gemm_f16_prepared(a.data_ptr(), b.bt.data_ptr(), out.data_ptr(), m, b.N, k, int(half),
+                                                 _stream()))
+        return out
+    b = _dev(b, "b", torch.float16, 2)
     k2, n = b.shape
     if k2 != k:
         raise ValueError(f"b: expected ({k}, N), got {tuple(b.shape)}")
-    half = out_dtype == "float16"
     out = torch.empty((m, n), dtype=torch.float16 if half else torch.float32, device=a.device)
     check(_lib.load().unit_gemm_f16(a.data_ptr(), b.data_ptr(), out.data_ptr(), m, n, k, int(half), _stream()))
     return out
