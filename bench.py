@@ -47,7 +47,7 @@ def main():
                          "or on the reference's blocked layout in every call")
     ap.add_argument("--profile", default=None, metavar="WHAT",
                     help="launch one kernel 20 times and exit (for rocprofv3): a ResNet-50 layer name such as "
-                         "3x3_256_256@14, or gemm_i8 / gemm_f16 / copy")
+                         "3x3_256_256@14, or gemm_i8 / gemm_f16 / gemm_f16_prepared / copy")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus must be 1 "
@@ -83,7 +83,7 @@ def main():
         torch.cuda.synchronize()
         return s.elapsed_time(e) * 1e3 / iters
 
-    if args.profile in ("gemm_i8", "gemm_f16", "copy"):
+    if args.profile in ("gemm_i8", "gemm_f16", "gemm_f16_prepared", "copy"):
         n = 4096
         if args.profile == "gemm_i8":
             a = dev_t(rng.uniform_u8((n, n), 11))
@@ -93,6 +93,10 @@ def main():
             a = dev_t(rng.normal_f16((n, n), 13, 1.0 / 64))
             b = dev_t(rng.normal_f16((n, n), 14))
             fn = lambda: U.gemm_fp16(a, b)
+        elif args.profile == "gemm_f16_prepared":
+            a = dev_t(rng.normal_f16((n, n), 13, 1.0 / 64))
+            pb = U.prepare_gemm_b(dev_t(rng.normal_f16((n, n), 14)))
+            fn = lambda: U.gemm_fp16(a, pb)
         else:  # plain 128 MiB device-to-device copy: the calibration point for FETCH_SIZE / WRITE_SIZE
             a = torch.empty(128 * 1024 * 1024, dtype=torch.uint8, device=dev)
             b = torch.empty_like(a)
