@@ -288,7 +288,7 @@ def main():
                                   max_rel_err=float((np.abs(got - ref) / np.maximum(np.abs(ref), 1e-3 * np.abs(ref).max())).max()))
 
     # ------------------------------------------------------------------ secondary legs (BASELINE configs 0, 3, 4-fp16, layouts)
-    def conv_i8_leg(shapes, batch, iters, fused=False, prepared=False):
+    def conv_i8_leg(shapes, batch, iters, fused=False, prepared=False, requant=False):
         rows, tot_us, tot_ops = [], 0.0, 0.0
         for i, s in enumerate(shapes):
             cb = WL.channel_block(s.C)
@@ -299,10 +299,15 @@ def main():
             o = torch.empty((batch, s.K // 16, oh, ow, 16), dtype=torch.int32, device=dev)
             desc = _lib.ConvDesc(batch, cp, s.H, s.W, s.K, s.KH, s.KW, s.stride, s.stride, s.pad, s.pad, s.pad, s.pad,
                                  1, 1, cb)
-            prep = prepared and (s.KH * s.KW <= 31 if cb == 16 else s.KW <= 8)
+            prep = (prepared or requant) and (s.KH * s.KW <= 31 if cb == 16 else s.KW <= 8)
             if prep:
                 w = U.prepare_conv2d_weight(w).buf
-            if fused:  # signed activations, bias and scale: the form the reference's quantized graphs run
+            if requant:  # u8 output in the layout the next convolution reads: 4 x less output traffic
+                o = torch.empty((batch, s.K // 16, oh, ow, 16), dtype=torch.uint8, device=dev)
+                bias = dev_t(rng.uniform_s8((s.K,), 5000 + i).astype(np.int32) * 1000)
+                f = lambda: _lib.check(L.unit_conv2d_nchwc_u8s8u8_requant_prepared(
+                    ctypes.byref(desc), d.data_ptr(), w.data_ptr(), bias.data_ptr(), 3, 14, o.data_ptr(), stream))
+            elif fused:  # signed activations, bias and scale: the form the reference's quantized graphs run
                 d = d.view(torch.int8)
                 bias = dev_t(rng.uniform_s8((s.K,), 5000 + i).astype(np.int32) * 1000)
                 fn = L.unit_conv2d_nchwc_s8s8s32_fused_prepared if prep else L.unit_conv2d_nchwc_s8s8s32_fused
@@ -333,6 +338,11 @@ def main():
     if use_prep:
         _, fr_us, _ = conv_i8_leg(WL.RESNET50, BATCH, 20, fused=True)
         fused_s8["reference_layout_weights_stack_us"] = round(fr_us, 1)
+    rq_rows, rq_us, rq_ops = conv_i8_leg(WL.RESNET50, BATCH, 20, requant=True)
+    requant_u8 = dict(workload="ResNet-50 v1 conv stack, batch 32, u8 x s8 with the output requantised to u8 NCHW16c "
+                               "(clamp(((conv + bias) * scale + half) >> shift, 0, 255)); an extension, not in the "
+                               "reference's graphs",
+                      stack_us=round(rq_us, 1), tops=round(rq_ops / rq_us / 1e6, 2), layers=rq_rows)
 
     # 3-D convolution workloads of apps/cpu/kernel/conv3d.py:13-25 (depth 16, batch 1)
     c3_rows = []
@@ -493,6 +503,7 @@ def main():
         "resnet18_b1": resnet18_b1,
         "conv_fp16_resnet50_b32": conv_fp16,
         "conv_fused_s8_resnet50_b32": fused_s8,
+        "conv_requant_u8_resnet50_b32": requant_u8,
         "conv3d_s8": conv3d,
         "layout_kernels": layout,
         "layers": table,

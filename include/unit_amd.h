@@ -223,6 +223,18 @@ int unit_conv2d_nchwc_s8s8s32_fused_prepared(const unit_conv_desc *d, const void
 int unit_conv2d_nchw16c_f16f32_prepared(const unit_conv_desc *d, const void *a, const void *prepared,
                                         void *out, unit_stream_t stream);
 
+/* u8 x s8 convolution on prepared weights with the output requantised to u8 in the blocked
+ * layout the next convolution reads, (N, K/16, OH, OW, 16) u8:
+ *   q = clamp(((conv_u8(data, w)[k] + bias[k]) * scale + 2^(shift-1)) >> shift, 0, 255)
+ * (sum and bias in int32, product and shift in 64 bits, 1 <= shift <= 62; the lower clamp is the
+ * ReLU).  bias: K int32 values or NULL.  Four times less output traffic than the int32 forms.
+ * No counterpart in the reference's files: its printed graphs stop at the int32
+ * subtract / add / multiply (apps/cpu/relay/result.log:15-24); this is the integer requantisation
+ * that follows it in a quantised network, defined here and by the oracle of the same name. */
+int unit_conv2d_nchwc_u8s8u8_requant_prepared(const unit_conv_desc *d, const void *data, const void *prepared,
+                                              const int32_t *bias, int32_t scale, int32_t shift, void *out,
+                                              unit_stream_t stream);
+
 /* ------------------------------------------------------------------ diagnostics */
 
 /* One v_mfma_i32_32x32x32_i8 / v_mfma_f32_32x32x16_f16 on a single wavefront, operands and

@@ -233,6 +233,25 @@ def conv2d_nchwc_int8_fused(data_s8, weight, bias, scale, stride=1, padding=0, d
     return np.ascontiguousarray((out & 0xFFFFFFFF).astype(np.uint32).view(np.int32))
 
 
+def conv2d_nchwc_u8_requant(data_u8, weight, bias, scale, shift, stride=1, padding=0, dilation=1, conv=None):
+    """u8 x s8 convolution with requantised u8 output (no counterpart in the reference's files: its
+    graphs stop at the int32 subtract / add / multiply, apps/cpu/relay/result.log:15-24; parity
+    unpinned beyond the convolution itself, which is pinned):
+
+        q = clamp(((conv_u8(x, w)[k] + bias[k]) * scale + 2**(shift - 1)) >> shift, 0, 255)
+
+    conv + bias in wrapping int32, product and arithmetic shift in 64 bits.  Output u8
+    (N, K/16, OH, OW, 16)."""
+    conv = conv or conv2d_nchwc_int8
+    acc = conv(np.asarray(data_u8), np.asarray(weight), stride, padding, dilation).astype(np.int64)
+    if bias is not None:
+        acc = acc + np.asarray(bias, dtype=np.int64).reshape(1, -1, 1, 1, 16)
+    acc = (acc & 0xFFFFFFFF).astype(np.uint32).view(np.int32).astype(np.int64)   # the int32 the device holds
+    assert 1 <= int(shift) <= 62
+    t = (acc * int(scale) + (1 << (int(shift) - 1))) >> int(shift)
+    return np.ascontiguousarray(np.clip(t, 0, 255).astype(np.uint8))
+
+
 def conv3d_ncdhwc_int8(data, weight, stride=1):
     """apps/cpu/kernel/conv3d.py:39-64, the reference's own te.compute: valid 3-D convolution, one
     stride, both operands int8 cast to int32:

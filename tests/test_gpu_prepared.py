@@ -293,3 +293,67 @@ def test_prepared_rejections(dev):
     with pytest.raises(ValueError):   # prepared for 4-channel blocks, data in 16-channel blocks
         p4 = U.prepare_conv2d_weight(_t(rng.uniform_s8((2, 4, 3, 3, 1, 16, 4), 1), dev))
         U.conv2d_NCHWc_int8(_t(rng.uniform_u8((1, 1, 8, 8, 16), 2), dev), p4, 1, 1)
+
+
+REQUANT_CASES = [
+    # N, C, H, W, K, kernel, stride, pad, scale, shift, with bias
+    (1, 64, 56, 56, 64, 3, 1, 1, 3, 12, True),
+    (2, 32, 9, 7, 48, 3, 1, 1, 1, 9, False),          # K not a multiple of 32: the last plane pair is half empty
+    (3, 64, 14, 14, 128, 1, 1, 0, -5, 11, True),      # negative scale
+    (1, 512, 7, 7, 512, 3, 1, 1, 77, 20, True),       # k-groups: partial tiles summed in LDS first
+    (2, 80, 9, 11, 96, 3, 2, (1, 0, 2, 1), 1 << 30, 45, True),   # 64-bit product and shift
+    (1, 4, 32, 32, 64, 7, 2, 3, 9, 12, True),         # 4-channel stem
+    (32, 64, 56, 56, 256, 1, 1, 0, 5, 13, True),      # ResNet-50 batch 32, output-bound layer
+    (1, 16, 8, 8, 16, 1, 1, 0, 1, 1, False),          # shift 1
+]
+
+
+@pytest.mark.parametrize("N,C,H,W,K,ks,stride,pad,scale,shift,with_bias", REQUANT_CASES)
+def test_conv2d_requant_u8(dev, oracle, N, C, H, W, K, ks, stride, pad, scale, shift, with_bias):
+    """Requantised u8 output against the oracle's integer definition (bit-exact), on inputs scaled so that the
+    results spread over the whole 0..255 range and both clamps."""
+    cb = 16 if C % 16 == 0 else 4
+    data = rng.uniform_u8((N, C // cb, H, W, cb), 7 * C + H)
+    wt = rng.uniform_s8((K // 16, C // cb, ks, ks, cb // 4, 16, 4), 3 * K + ks)
+    bias = rng.uniform_s8((K,), 5).astype(np.int32) * 20011 if with_bias else None
+    ref = oracle.conv2d_nchwc_u8_requant(data, wt, bias, scale, shift, stride, pad, 1, conv=oracle.c_conv2d_nchwc)
+    out = U.conv2d_NCHWc_int8_requant(_t(data, dev), U.prepare_conv2d_weight(_t(wt, dev)),
+                                      _t(bias, dev) if with_bias else None, scale, shift, stride, pad)
+    torch.cuda.synchronize()
+    assert U.last_variant().startswith("q8prep")
+    assert out.dtype == torch.uint8 and tuple(out.shape) == ref.shape
+    got = out.cpu().numpy()
+    assert np.array_equal(got, ref), U.last_variant()
+
+
+def test_conv2d_requant_every_direct_variant(dev, oracle, monkeypatch):
+    from unit_amd import _lib
+    N, C, H, W, K, ks = 2, 80, 9, 11, 96, 3
+    data = rng.uniform_u8((N, C // 16, H, W, 16), 41)
+    wt = rng.uniform_s8((K // 16, C // 16, ks, ks, 4, 16, 4), 42)
+    bias = rng.uniform_s8((K,), 43).astype(np.int32) * 3001
+    ref = oracle.conv2d_nchwc_u8_requant(data, wt, bias, 7, 13, 1, 1, 1, conv=oracle.c_conv2d_nchwc)
+    assert 0 < (ref == 0).mean() < 0.9 and (ref == 255).any()   # both clamps and the range in between occur
+    d, tb = _t(data, dev), _t(bias, dev)
+    p = U.prepare_conv2d_weight(_t(wt, dev))
+    names = set()
+    for v in range(1, _lib.load().unit_conv_variant_count() + 1):
+        monkeypatch.setenv("UNIT_AMD_CONV_VARIANT", str(v))
+        out = U.conv2d_NCHWc_int8_requant(d, p, tb, 7, 13, 1, 1)
+        torch.cuda.synchronize()
+        names.add(U.last_variant())
+        assert np.array_equal(out.cpu().numpy(), ref), (v, U.last_variant())
+    assert len(names) >= 15
+
+
+def test_conv_chain_through_requantised_activations(dev, oracle):
+    """Two layers back to back: the u8 output of the first is the input of the second, no layout change."""
+    x = rng.uniform_u8((2, 4, 12, 12, 16), 51)
+    w1 = rng.uniform_s8((8, 4, 3, 3, 4, 16, 4), 52)
+    w2 = rng.uniform_s8((4, 8, 1, 1, 4, 16, 4), 53)
+    mid_ref = oracle.conv2d_nchwc_u8_requant(x, w1, None, 3, 14, 1, 1, 1, conv=oracle.c_conv2d_nchwc)
+    ref = oracle.c_conv2d_nchwc(mid_ref, w2, 1, 0, 1)
+    mid = U.conv2d_NCHWc_int8_requant(_t(x, dev), _t(w1, dev), None, 3, 14, 1, 1)
+    out = U.conv2d_NCHWc_int8(mid, U.prepare_conv2d_weight(_t(w2, dev)), 1, 0)
+    torch.cuda.synchronize()
+    assert np.array_equal(mid.cpu().numpy(), mid_ref) and np.array_equal(out.cpu().numpy(), ref)

@@ -308,3 +308,24 @@ def test_fp16_conv_matches_torch_double(oracle):
         out5 = oracle.conv2d_nchw16c_f16(oracle.pack_nchwc(x, 16), oracle.prepack_conv_weight_f16(w), st, st)
         ref = torch.nn.functional.conv2d(torch.from_numpy(x).double(), torch.from_numpy(w).double(), stride=st).numpy()
         assert np.allclose(oracle.unpack_nchwc(out5), ref, rtol=1e-12, atol=1e-12)
+
+
+def test_requant_definition_small_cases(oracle):
+    """The integer requantisation, spelled out scalar by scalar with Python integers on a tiny case
+    (floor shift of the 64-bit product plus half, both clamps), and the identities that fix its
+    corners: shift s with scale 2**s gives round-half-up of conv + bias clamped; a negative
+    accumulator always gives 0."""
+    x = oracle.fill_u8((1, 1, 5, 5, 16), 71)
+    w = oracle.fill_s8((1, 1, 3, 3, 4, 16, 4), 72)
+    bias = (np.arange(16, dtype=np.int32) - 8) * 3000
+    acc = oracle.conv2d_nchwc_int8(x, w, 1, 1, 1).astype(np.int64) + bias.reshape(1, 1, 1, 1, 16)
+    for scale, shift in ((3, 10), (-2, 7), (1 << 20, 36), (1, 1)):
+        got = oracle.conv2d_nchwc_u8_requant(x, w, bias, scale, shift, 1, 1, 1)
+        want = np.zeros(acc.shape, np.uint8)
+        for idx in np.ndindex(*acc.shape):
+            t = (int(acc[idx]) * scale + (1 << (shift - 1))) >> shift   # Python ints: exact, floor shift
+            want[idx] = min(255, max(0, t))
+        assert np.array_equal(got, want)
+    ident = oracle.conv2d_nchwc_u8_requant(x, w, bias, 1 << 8, 16, 1, 1, 1)   # (acc * 256 + 2**15) >> 16 = round(acc / 256)
+    assert np.array_equal(ident, np.clip(np.floor(acc / 256.0 + 0.5), 0, 255).astype(np.uint8))
+    assert (oracle.conv2d_nchwc_u8_requant(x, w, bias, 5, 3, 1, 1, 1)[acc < -1] == 0).all()

@@ -36,6 +36,7 @@ SYMBOLS = (
     "unit_conv2d_nchwc_u8s8s32_prepared",
     "unit_conv2d_nchwc_s8s8s32_fused_prepared",
     "unit_conv2d_nchw16c_f16f32_prepared",
+    "unit_conv2d_nchwc_u8s8u8_requant_prepared",
     "unit_mfma_tile_i8",
     "unit_mfma_tile_f16",
     "unit_mfma_peak",
@@ -96,6 +97,7 @@ def load():
     L.unit_conv2d_nchwc_u8s8s32_prepared.argtypes = [dp, vp, vp, vp, vp]
     L.unit_conv2d_nchwc_s8s8s32_fused_prepared.argtypes = [dp, vp, vp, vp, i32, vp, vp]
     L.unit_conv2d_nchw16c_f16f32_prepared.argtypes = [dp, vp, vp, vp, vp]
+    L.unit_conv2d_nchwc_u8s8u8_requant_prepared.argtypes = [dp, vp, vp, vp, i32, i32, vp, vp]
     L.unit_mfma_tile_i8.argtypes = [vp, vp, vp, vp]
     L.unit_mfma_tile_f16.argtypes = [vp, vp, vp, vp]
     L.unit_mfma_peak.argtypes = [i32, i32, i32, vp, vp]

@@ -111,7 +111,71 @@ __device__ __forceinline__ void store_block(const typename ConvEpilogue<Op>::Par
   }
 }
 
-template <class Op, class S, bool SHIFT, bool PREP = false, bool C4 = false>
+// Requantised output: one 32-channel x 32-pixel int32 block -> u8 (N, K/16, OH, OW, 16),
+//   q = clamp(((acc + addend[c]) * scale + 2^(shift-1)) >> shift, 0, 255)
+// with the product and the shift in 64 bits.  A lane holds 16 channels of one pixel (4 h + 8 q + e);
+// after packing each quad into a dword the two 32-lane halves swap two dwords each, so that half h
+// holds the 16 bytes of plane c0 / 16 + h of its pixel: one 16-byte store per lane, 512 consecutive
+// bytes per plane, no LDS.
+template <class Op>
+__device__ __forceinline__ void store_block_q8(const typename ConvEpilogue<Op>::Params &p, const v16i &acc, const int *wsb,
+                                               int c0, int m0, int lane) {
+  const int l32 = lane & 31, half = lane >> 5;
+  int d[4];
+  if (p.shift >= 33) {
+    // The rounding term 2^(shift-1) is a multiple of 2^32, so it and the shift act on the high
+    // dword of the product alone: floor((hi * 2^32 + lo + R) / 2^shift) = (hi + R / 2^32) >> (shift - 32).
+    // (The host doubles scale and increments shift while that keeps scale in int32 -- the same
+    // rational number -- so practical shifts arrive here.)
+    const int rhi = 1 << (p.shift - 33), sh = p.shift - 32;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      u32 packed = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        int v = acc[4 * q + e];
+        if (wsb) v += wsb[8 * q + 4 * half + e];
+        int t = min(max((__mulhi(v, p.scale) + rhi) >> sh, 0), 255);
+        // Opaque to the optimiser on purpose: left visible, shift + clamp + pack of two values is
+        // matched to v_ashr_pk_u8_i32, whose result this compiler treats as zero-extended while
+        // the upper 16 bits of the destination came back non-zero (bytes 2 and 3 of the packed
+        // dword read 255 whenever the first value was negative before the shift).
+        asm volatile("" : "+v"(t));
+        packed |= (u32)t << (8 * e);
+      }
+      d[q] = (int)packed;
+    }
+  } else {
+    const long long rnd = 1ll << (p.shift - 1);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      u32 packed = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        int v = acc[4 * q + e];
+        if (wsb) v += wsb[8 * q + 4 * half + e];
+        long long t = ((long long)v * p.scale + rnd) >> p.shift;
+        t = t < 0 ? 0 : (t > 255 ? 255 : t);
+        packed |= (u32)t << (8 * e);
+      }
+      d[q] = (int)packed;
+    }
+  }
+  // half 0 keeps d0, d1 (channels 0-3, 8-11) and needs the partner's d0, d1 (4-7, 12-15);
+  // half 1 keeps d2, d3 (20-23, 28-31) and needs the partner's d2, d3 (16-19, 24-27)
+  const int s0 = half ? d[0] : d[2], s1 = half ? d[1] : d[3];
+  const int r0 = __shfl_xor(s0, 32), r1 = __shfl_xor(s1, 32);
+  const v4i row = half ? v4i{r0, d[2], r1, d[3]} : v4i{d[0], r0, d[1], r1};
+  const int m = m0 + l32, c = c0 + half * 16;
+  if (c < p.K && m < p.npix) {
+    int n, pix;
+    p.by_ohw.divmod(m, n, pix);
+    char *dst = static_cast<char *>(p.out) + (((size_t)n * (p.K >> 4) + (c >> 4)) * p.ohw + pix) * 16;
+    __builtin_nontemporal_store(row, reinterpret_cast<v4i *>(dst));
+  }
+}
+
+template <class Op, class S, bool SHIFT, bool PREP = false, bool C4 = false, bool Q8 = false>
 __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ data, const char *__restrict__ wgt,
                                                      typename ConvEpilogue<Op>::Params ep, ConvGeom g, GridMap gm) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -121,6 +185,7 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
   constexpr int WTAP = kInt ? 256 : 512;           // bytes of one tap of a 16-channel weight block
   static_assert(kInt || (!SHIFT && !S::PAD), "the fp16 operator has neither a shift nor padding");
   static_assert(!C4 || (kInt && S::PAD), "4-channel blocks: int8, masked loads");
+  static_assert(!Q8 || kInt, "requantised output is an int8 operator");
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int l32 = lane & 31, half = lane >> 5;
@@ -195,6 +260,9 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
     if constexpr (kInt) {
       const int c = x0 + i * 32 + l32;
       if (ep.bias != nullptr && wave == 0 && c < ep.K) addv[i] = ep.bias[c];
+      if constexpr (Q8) {
+        if (ep.bias2 != nullptr && wave == 0 && c < ep.K) addv[i] += ep.bias2[c];
+      }
     }
   }
   // data: byte offset of the window origin of this lane's pixel per 32-pixel block, and the set of
@@ -397,7 +465,7 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
   }
   // what is added per channel before the scale: the shift correction and / or the bias; one wave
   // adds the bias.  `addend` is uniform over the workgroup.
-  const bool addend = kInt && (SHIFT || ep.bias != nullptr);
+  const bool addend = kInt && (SHIFT || ep.bias != nullptr || (Q8 && ep.bias2 != nullptr));
 #pragma unroll
   for (int i = 0; i < TX; ++i) wsx[i] += addv[i];
 
@@ -410,8 +478,11 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
     for (int i = 0; i < TX; ++i)
 #pragma unroll
       for (int j = 0; j < TY; ++j)
-        store_block<Op>(ep, acc[i][j], addend ? wsum + i * 32 : nullptr, ep.scale, x0 + i * 32, y0 + j * 32, lane,
-                        scratch);
+        if constexpr (Q8)
+          store_block_q8<Op>(ep, acc[i][j], addend ? wsum + i * 32 : nullptr, x0 + i * 32, y0 + j * 32, lane);
+        else
+          store_block<Op>(ep, acc[i][j], addend ? wsum + i * 32 : nullptr, ep.scale, x0 + i * 32, y0 + j * 32, lane,
+                          scratch);
   } else if constexpr (!kParked) {
     // sum the partial tiles of the KG waves in LDS, then share the blocks among the waves
     int *sum = reinterpret_cast<int *>(tiles);
@@ -434,7 +505,10 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
       v16i total;
 #pragma unroll
       for (int r = 0; r < 16; ++r) total[r] = sum[(b * 16 + r) * 64 + lane];
-      store_block<Op>(ep, total, addend ? wsum + i * 32 : nullptr, ep.scale, x0 + i * 32, y0 + j * 32, lane, scratch);
+      if constexpr (Q8)
+        store_block_q8<Op>(ep, total, addend ? wsum + i * 32 : nullptr, x0 + i * 32, y0 + j * 32, lane);
+      else
+        store_block<Op>(ep, total, addend ? wsum + i * 32 : nullptr, ep.scale, x0 + i * 32, y0 + j * 32, lane, scratch);
     }
   } else {
     // every wave parks its partial tile (and addends); the owner of a block adds them in wave order

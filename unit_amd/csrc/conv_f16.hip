@@ -25,7 +25,7 @@ int run_conv_f16(const unit_conv_desc *d, const ConvGeom &g0, const void *a, con
   // weight element (ko, tap, i, o): ((ko * ntaps + tap) * 16 + i) * 16 + o  -> k = tap*16 + i
   typename XL::Params xp{static_cast<const char *>(b), d->K, g.ntaps * 16, 16, (size_t)g.ntaps * 512, 32};
   typename YL::Params yp{static_cast<const char *>(a), g};
-  typename Epi::Params ep{out, d->K, g.OH * g.OW, g.npix, g.by_ohw, nullptr, 1};
+  typename Epi::Params ep{out, d->K, g.OH * g.OW, g.npix, g.by_ohw, nullptr, 1, nullptr, 0};
   const int gx = ceil_div(d->K, T::BX), gy = ceil_div(g.npix, T::BY);
   const int panel = plan.panel > 0 && plan.panel < gx ? plan.panel : 0;
   char tail[16] = "";

@@ -22,7 +22,7 @@ int run_conv_i8(const unit_conv_desc *d, const ConvGeom &g0, const void *data, c
   g.ntab = nk * T::BKB / TAPB;
   typename XL::Params xp{static_cast<const char *>(w), d->K, kbytes / 4};
   typename YL::Params yp{static_cast<const char *>(data), g};
-  typename Epi::Params ep{out, d->K, g.OH * g.OW, g.npix, g.by_ohw, bias, scale};
+  typename Epi::Params ep{out, d->K, g.OH * g.OW, g.npix, g.by_ohw, bias, scale, nullptr, 0};
   const char *what = SIGNED ? "unit_conv2d_nchwc_s8s8s32_fused" : "unit_conv2d_nchwc_u8s8s32";
   const int gx = ceil_div(d->K, T::BX), gy = ceil_div(g.npix, T::BY);
   const int splits = plan.splits > nk ? nk : plan.splits;

@@ -17,6 +17,8 @@ int conv_s8_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGe
                      const int *bias, int scale, void *out, hipStream_t s);  // conv_prepared_s8.hip
 int conv_c4_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
                      const int *addend, int scale, bool shift, void *out, hipStream_t s);  // conv_prepared_c4.hip
+int conv_q8_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
+                     const int *addend, const int *bias, int scale, int shift, void *out, hipStream_t s);  // conv_prepared_q8.hip
 int conv_f16_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *a, const void *w,
                       void *out, hipStream_t s);  // conv_prepared_f16.hip
 
@@ -194,6 +196,29 @@ extern "C" int unit_conv2d_nchwc_u8s8s32_prepared(const unit_conv_desc *d, const
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (d->cb == 4) return conv_c4_prepared(p, d, g, data, w, addend, 1, true, out, s);
   return conv_u8_prepared(p, d, g, data, w, addend, out, s);
+}
+
+extern "C" int unit_conv2d_nchwc_u8s8u8_requant_prepared(const unit_conv_desc *d, const void *data, const void *prepared,
+                                                         const int32_t *bias, int32_t scale, int32_t shift, void *out,
+                                                         unit_stream_t stream) {
+  using namespace unit;
+  const char *what = "unit_conv2d_nchwc_u8s8u8_requant_prepared";
+  if (!d || !data || !prepared || !out) return fail(UNIT_E_ARG, "%s: null pointer", what);
+  if (shift < 1 || shift > 62) return fail(UNIT_E_ARG, "%s: shift must be in 1..62 (got %d)", what, shift);
+  ConvGeom g;
+  if (int rc = check_prepared_conv(what, d, 16, &g, data, prepared, out)) return rc;
+  const PreparedLayout pl = prepared_layout(d->K, d->C, d->KH, d->KW, d->cb, 1);
+  const int ntable = (int)(sizeof(kTunedI8Prepared) / sizeof(kTunedI8Prepared[0])) - 1;
+  const ConvPlan p = plan_prepared(d, g, g.ntaps * d->cb, kTunedI8Prepared, ntable, true);
+  const char *w = static_cast<const char *>(prepared);
+  // (v * scale + 2^(shift-1)) >> shift is unchanged when scale doubles and shift grows by one; with
+  // shift >= 33 the kernel needs only the high dword of the product
+  while (shift < 33 && scale >= -(1 << 30) && scale < (1 << 30)) {
+    scale *= 2;
+    ++shift;
+  }
+  return conv_q8_prepared(p, d, g, data, w, reinterpret_cast<const int *>(w + pl.frag_bytes), bias, scale, shift, out,
+                          static_cast<hipStream_t>(stream));
 }
 
 extern "C" int unit_conv2d_nchwc_s8s8s32_fused_prepared(const unit_conv_desc *d, const void *data,

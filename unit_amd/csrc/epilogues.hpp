@@ -74,6 +74,9 @@ struct ConvEpilogue {
     // fused int8 form (apps/cpu/relay/result.log:17-20): out = (acc + bias[channel]) * scale
     const int *bias;  // K values or null
     int scale;
+    // requantised u8 output (direct kernels, Q8): a second per-channel addend and the right shift
+    const int *bias2;
+    int shift;
   };
   static constexpr int kPitch = 144;               // bytes per pixel row of the scratch
   static constexpr int kScratch = 32 * kPitch;     // per wave

@@ -22,6 +22,7 @@ __all__ = [
     "pack_nchwc", "unpack_nchwc", "prepack_conv_weight", "prepack_dense_weight",
     "prepack_conv_weight_f16", "conv_out_hw", "last_variant",
     "PreparedConvWeight", "prepare_conv2d_weight", "PreparedGemmB", "prepare_gemm_b",
+    "conv2d_NCHWc_int8_requant",
 ]
 
 
@@ -246,6 +247,48 @@ def conv2d_NCHWc_int8_fused(data, kernel, bias, scale, stride, padding, dilation
     fn = L.unit_conv2d_nchwc_s8s8s32_fused_prepared if prepared else L.unit_conv2d_nchwc_s8s8s32_fused
     check(fn(ctypes.byref(d), data.data_ptr(), kernel.buf.data_ptr() if prepared else kernel.data_ptr(),
              bias.data_ptr() if bias is not None else None, scale, out.data_ptr(), _stream()))
+    return out
+
+
+def conv2d_NCHWc_int8_requant(data, kernel, bias, scale, shift, stride, padding, dilation=1):
+    """u8 x s8 convolution whose output is requantised to u8 in the blocked layout the next
+    convolution reads (four times less output traffic than int32):
+
+        q = clamp(((conv(data, kernel)[k] + bias[k]) * scale + 2**(shift - 1)) >> shift, 0, 255)
+
+    data   uint8 (N, C/cb, H, W, cb)
+    kernel a PreparedConvWeight (prepare_conv2d_weight), or the blocked int8 kernel (prepared here)
+    bias   int32 (K,) or None;  scale int32;  shift 1..62
+    returns uint8 (N, K/16, OH, OW, 16)
+
+    The reference's graphs stop at the int32 subtract / add / multiply
+    (apps/cpu/relay/result.log:15-24); this is the integer requantisation that follows it in a
+    quantised network.
+    """
+    import ctypes
+    data = _dev(data, "data", torch.uint8, 5)
+    if not isinstance(kernel, PreparedConvWeight):
+        kernel = prepare_conv2d_weight(kernel)
+    n, cc, h, w, cb = data.shape
+    ko, _, kh, kw = _prepared_dims(kernel, data, torch.int8)
+    if bias is not None:
+        if bias.dtype != torch.int32 or bias.numel() != ko * 16 or bias.device != data.device:
+            raise ValueError(f"bias: expected {ko * 16} int32 values on {data.device}")
+        bias = bias.contiguous()
+    scale, shift = int(scale), int(shift)
+    if not -2 ** 31 <= scale < 2 ** 31:
+        raise ValueError("scale: must fit int32")
+    sh, sw = _pair(stride, "stride")
+    dh, dw = _pair(dilation, "dilation")
+    pt, pl, pb, pr = _pad4(padding)
+    d = ConvDesc(n, cc * cb, h, w, ko * 16, kh, kw, sh, sw, pt, pl, pb, pr, dh, dw, cb)
+    L = _lib.load()
+    oh, ow = ctypes.c_int32(), ctypes.c_int32()
+    check(L.unit_conv_out_hw(ctypes.byref(d), ctypes.byref(oh), ctypes.byref(ow)))
+    out = torch.empty((n, ko, oh.value, ow.value, 16), dtype=torch.uint8, device=data.device)
+    check(L.unit_conv2d_nchwc_u8s8u8_requant_prepared(ctypes.byref(d), data.data_ptr(), kernel.buf.data_ptr(),
+                                                      bias.data_ptr() if bias is not None else None, scale, shift,
+                                                      out.data_ptr(), _stream()))
     return out
 
 
