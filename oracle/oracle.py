@@ -13,6 +13,11 @@ Parity status:
   * dense packed-weight *index order*: PARITY UNPINNED -- the reference gives only the
     placeholder shape (N/128, K/4, 128, 4) (apps/cpu/kernel/int8-gemm.py:14) and never
     checks values through it.  The logical product a . W^T is pinned.
+  * fused signed form with spatial padding: PARITY UNPINNED (the reference's printed graphs have
+    padding 0; zero padding of the signed data follows upstream TVM).
+  * conv2d_nchwc_u8_requant: PARITY UNPINNED -- an extension with no counterpart in the
+    reference (its graphs stop at the int32 subtract / add / multiply); the convolution inside is
+    the pinned one, the requantisation is checked against exact Python integers.
 """
 import ctypes
 import os
