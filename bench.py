@@ -287,7 +287,7 @@ def main():
                                   pct_f16_peak=round(100 * gemm_ops / us_fp / 1e6 / PEAK_F16_TFLOPS, 2), kernel=v_fp,
                                   max_rel_err=float((np.abs(got - ref) / np.maximum(np.abs(ref), 1e-3 * np.abs(ref).max())).max()))
 
-    # ------------------------------------------------------------------ secondary legs (BASELINE configs 0, 3, 4-fp16, layouts)
+    # ------------------------------------------------------------------ secondary legs (BASELINE.json configs 0, 3, 4-fp16; layouts)
     def conv_i8_leg(shapes, batch, iters, fused=False, prepared=False, requant=False):
         rows, tot_us, tot_ops = [], 0.0, 0.0
         for i, s in enumerate(shapes):
@@ -325,10 +325,10 @@ def main():
 
     use_prep = args.weights == "prepared"
     r18_rows, r18_us, r18_ops = conv_i8_leg(WL.RESNET18, 1, 30, prepared=use_prep)
-    resnet18_b1 = dict(workload="ResNet-18 v1 conv layers, batch 1, int8 (BASELINE configs[3])",
+    resnet18_b1 = dict(workload="ResNet-18 v1 conv layers, batch 1, int8 (BASELINE.json configs[3])",
                        stack_us=round(r18_us, 1), tops=round(r18_ops / r18_us / 1e6, 2), layers=r18_rows)
     single_rows, _, _ = conv_i8_leg((WL.SINGLE_CONV,), 1, 50, prepared=use_prep)
-    single_conv = dict(workload="N=1 C=64 56x56 K=64 3x3 s1 p1 NCHW16c (BASELINE configs[0])", **single_rows[0],
+    single_conv = dict(workload="N=1 C=64 56x56 K=64 3x3 s1 p1 NCHW16c (BASELINE.json configs[0])", **single_rows[0],
                        reference_us=24.27, reference_source="cpu-tune.log:160 (x86 VNNI, hardware unstated)")
 
     fu_rows, fu_us, fu_ops = conv_i8_leg(WL.RESNET50, BATCH, 20, fused=True, prepared=use_prep)
@@ -389,7 +389,7 @@ def main():
                              pct_f16_peak=round(100 * flops / us / 1e6 / PEAK_F16_TFLOPS, 2), kernel=U.last_variant()))
         f16_us += us * s.count
         f16_flops += flops * s.count
-    conv_fp16 = dict(workload="ResNet-50 v1 conv layers except the stem, batch 32, fp16 -> fp32 (BASELINE configs[4], "
+    conv_fp16 = dict(workload="ResNet-50 v1 conv layers except the stem, batch 32, fp16 -> fp32 (BASELINE.json configs[4], "
                               "fp16 variant)", stack_us=round(f16_us, 1), tflops=round(f16_flops / f16_us / 1e6, 1),
                      layers=f16_rows)
     if use_prep:
@@ -481,7 +481,7 @@ def main():
         "dtype": "u8",
         "data": "synthetic",
         "config": {"workload": "ResNet-50 v1 conv stack (53 convolutions, 20 unique shapes), batch 32, int8 "
-                               "u8 x s8 -> i32, NCHW16c / NCHW4c stem (BASELINE configs[4])",
+                               "u8 x s8 -> i32, NCHW16c / NCHW4c stem (BASELINE.json configs[4])",
                    "batch": BATCH, "ops_per_step": step_ops,
                    "weights": ("prepared once before the timed region (unit_conv2d_prepare_weight: MFMA fragment "
                                "order + 128 * sum(w)), as the reference folds its weight layout chain and sum(w) "

@@ -1,5 +1,5 @@
 """Parity of the fp16 HIP path against a float64 reference on the fp16-rounded inputs.
-Tolerance (BASELINE north star): max |d| / max(|ref|, eps * max|ref|) <= 1e-2."""
+Tolerance of the fp16 path: max |d| / max(|ref|, eps * max|ref|) <= 1e-2."""
 import numpy as np
 import pytest
 import torch

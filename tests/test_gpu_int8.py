@@ -99,7 +99,7 @@ def test_dense_extremes(dev, oracle):
 
 CONV_CASES = [
     # N, C, H, W, K, kernel, stride, pad, dilation
-    (1, 64, 56, 56, 64, 3, 1, 1, 1),       # BASELINE config (1)
+    (1, 64, 56, 56, 64, 3, 1, 1, 1),       # the single-convolution benchmark configuration
     (2, 32, 9, 7, 32, 3, 1, 1, 1),         # tiny, ragged pixel count
     (1, 16, 8, 8, 48, 1, 2, 0, 1),         # 1x1 stride 2, K not a multiple of 32
     (3, 64, 14, 14, 128, 1, 1, 0, 1),      # 1x1 = GEMM
@@ -308,7 +308,7 @@ def test_dense_golden_fixtures(dev, path):
 
 
 def test_full_size_properties(dev):
-    """BASELINE-size checks that need no CPU reference: 4096^3 int8 GEMM and a batch-32 ResNet-50
+    """Benchmark-size checks that need no CPU reference: 4096^3 int8 GEMM and a batch-32 ResNet-50
     layer through size-independent properties (linearity in the weights, the packed and un-packed
     weight paths agree, all-ones weights give per-row activation sums)."""
     M = N = K = 4096

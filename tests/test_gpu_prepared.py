@@ -92,7 +92,7 @@ def test_prepared_buffer_fp16(dev, K, C, ks):
 
 CONV_CASES = [
     # N, C, H, W, K, kernel, stride, pad, dilation
-    (1, 64, 56, 56, 64, 3, 1, 1, 1),       # BASELINE config (1)
+    (1, 64, 56, 56, 64, 3, 1, 1, 1),       # the single-convolution benchmark configuration
     (2, 32, 9, 7, 32, 3, 1, 1, 1),         # tiny, ragged pixel count
     (1, 16, 8, 8, 48, 1, 2, 0, 1),         # one tap (half a k-step), K not a multiple of 32
     (1, 16, 9, 9, 48, 3, 1, 0, 1),         # 9 taps, no padding: the kernel without tap masks on an odd tap count

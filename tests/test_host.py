@@ -48,7 +48,7 @@ def test_workloads():
     assert len(WL.RESNET18) == 11 and len(WL.RESNET50) == 20
     assert sum(s.count for s in WL.RESNET50) == 53 and sum(s.count for s in WL.RESNET18) == 20
     s = WL.SINGLE_CONV
-    assert WL.macs(s, 1) == 115605504  # 115.6 M MAC for BASELINE config (1)
+    assert WL.macs(s, 1) == 115605504  # 115.6 M MAC for the single-convolution benchmark configuration
     assert WL.algorithmic_bytes(s, 1) == 200704 + 36864 + 802816
     stem = WL.RESNET50[0]
     assert WL.channel_block(stem.C) == 4 and WL.channel_block(64) == 16
