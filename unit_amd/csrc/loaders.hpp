@@ -166,6 +166,7 @@ struct KMajorF16Loader {
   static constexpr int CPR = BKB / 16, QUADS = ROWS / 4, UNITS = QUADS * CPR;
   static constexpr int UPT = (UNITS + NT - 1) / NT;
   static constexpr bool kAllActive = UNITS % NT == 0;  // else UNITS < NT: threads >= UNITS idle
+  static constexpr int kLoads = UPT * 8;               // global loads per thread and stage
   static_assert(kAllActive || UNITS < NT, "k-major loader shape");
 
   v2i r[PF][UPT][8];

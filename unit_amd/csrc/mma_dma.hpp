@@ -202,3 +202,145 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
 }
 
 }  // namespace unit
+
+namespace unit {
+
+// Hybrid of the two pipelines: the X operand (K-contiguous rows) goes global -> LDS directly
+// through a two-buffer ring, the Y operand through a register loader (YRL: fetch to registers,
+// commit to LDS), for operands that have to be transposed on the way (the fp16 GEMM's b (K, N)).
+//
+// Stage kt computes from buffer kt % 2.  Y(kt + 2) is fetched into registers at the start of stage
+// kt and committed into the same buffer right after the barrier that ends the reads of stage kt;
+// X(kt + 2) is issued there too.  vmcnt accounting: when the barrier of stage kt is reached the
+// outstanding loads are X(kt + 1) (older) and the Y(kt + 2) fetches (younger, YRL::kLoads of them).
+template <class Op, class T, class YRL, class Epi>
+__global__ __launch_bounds__(T::NT) void mma_hybrid_kernel(DmaParams p, typename YRL::Params yp, typename Epi::Params ep,
+                                                           int nk, GridMap gm) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  const int t = threadIdx.x;
+  const int lane = t & 63, wave = t >> 6;
+  const int wx = wave % T::WX, wy = wave / T::WX;
+  const int l32 = lane & 31, half = lane >> 5;
+  constexpr int KK = T::BKB / 32, CPR = T::CPR, NW = T::NT / 64;
+  constexpr int RPL = 64 / CPR;
+  constexpr int XL = T::BX / RPL / NW;
+  static_assert(T::BX % (RPL * NW) == 0 && KK % 2 == 0 && YRL::kPF == 1, "hybrid kernel shape");
+  constexpr int NM = T::TX * T::TY, NF = T::TX + T::TY;
+  static_assert(NM >= XL && NM >= NF, "not enough MFMAs per k-step to carry the step's other work");
+
+  int bx, by, split;
+  gm.locate(blockIdx.x, bx, by, split);
+  const int x0 = bx * T::BX, y0 = by * T::BY;
+
+  u32 xoff[XL];
+  const int lrow = lane / CPR, slot = lane % CPR;
+#pragma unroll
+  for (int i = 0; i < XL; ++i) {
+    const int row = (wave * XL + i) * RPL + lrow;
+    int g = x0 + row;
+    g = g < p.xrows ? g : p.xrows - 1;
+    xoff[i] = (u32)g * (u32)p.ld + ((slot ^ swz<T::BKB>(row)) << 4);
+  }
+  YRL yl;
+  yl.init(yp, y0, t, nullptr);
+
+  auto issue_one = [&](int kt, int i) {
+    char *buf = lds + (kt & 1) * T::STAGE;
+    const char *xs = p.x + (size_t)kt * T::BKB;
+    __builtin_amdgcn_global_load_lds((gptr_t)(xs + xoff[i]), (lptr_t)(buf + (wave * XL + i) * 1024), 16, 0, 0);
+  };
+
+  typename Op::acc_t acc[T::TX][T::TY];
+#pragma unroll
+  for (int i = 0; i < T::TX; ++i)
+#pragma unroll
+    for (int j = 0; j < T::TY; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+  int wsx[T::TX], wsy[T::TY];
+#pragma unroll
+  for (int i = 0; i < T::TX; ++i) wsx[i] = 0;
+#pragma unroll
+  for (int j = 0; j < T::TY; ++j) wsy[j] = 0;
+
+  const int xrow = wx * (T::TX * 32) + l32, yrow = wy * (T::TY * 32) + l32;
+  const int xsw = swz<T::BKB>(xrow), ysw = swz<T::BKB>(yrow);
+  const int xbase = xrow * T::BKB, ybase = T::XBYTES + yrow * T::BKB;
+
+  v4i xf[2][T::TX], yf[2][T::TY];
+  auto load_one = [&](const char *stage, int kk, int s, int idx) {
+    const int cx = ((2 * kk + half) ^ xsw) << 4, cy = ((2 * kk + half) ^ ysw) << 4;
+    if (idx == 0)
+      xf[s][0] = *reinterpret_cast<const v4i *>(stage + xbase + cx);
+    else if (idx <= T::TY)
+      yf[s][idx - 1] = *reinterpret_cast<const v4i *>(stage + ybase + (idx - 1) * 32 * T::BKB + cy);
+    else
+      xf[s][idx - T::TY] = *reinterpret_cast<const v4i *>(stage + xbase + (idx - T::TY) * 32 * T::BKB + cx);
+  };
+  // one k-step: MFMAs with one slice of other work after each
+  auto step = [&](int s, const char *rd_stage, int rd_kk, int issue_kt, auto has_read, auto has_issue) {
+#pragma unroll
+    for (int m = 0; m < NM; ++m) {
+      const int i = m / T::TY, j = m % T::TY;
+      acc[i][j] = Op::mma(xf[s][i], yf[s][j], acc[i][j]);
+      if constexpr (decltype(has_read)::value) {
+        if (m < NF) load_one(rd_stage, rd_kk, s ^ 1, m);
+      }
+      if constexpr (decltype(has_issue)::value) {
+        if (m >= NM - XL) issue_one(issue_kt, m - (NM - XL));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  using yes = std::integral_constant<bool, true>;
+  using no = std::integral_constant<bool, false>;
+
+  // AHEAD: stage kt + 2 exists (fetched at the start, committed / issued after the barrier);
+  // NEXT: stage kt + 1 exists
+  auto stage = [&](int kt, auto ahead, auto next) {
+    const char *cur = lds + (kt & 1) * T::STAGE;
+    char *other = lds + ((kt + 1) & 1) * T::STAGE;
+    if constexpr (decltype(ahead)::value) yl.template fetch<0>(kt + 2);
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      if (kk + 1 < KK) {
+        step(kk & 1, cur, kk + 1, -1, yes{}, no{});
+      } else {
+        // X(kt + 1) must have landed; the Y(kt + 2) fetches may stay in flight
+        if constexpr (decltype(ahead)::value)
+          UNIT_WAIT_VMCNT(YRL::kLoads);
+        else
+          UNIT_WAIT_VMCNT(0);
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's reads of `cur` are done
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (decltype(ahead)::value) yl.template commit<0>(const_cast<char *>(cur) + T::XBYTES);
+        step(kk & 1, other, 0, kt + 2, next, ahead);
+      }
+    }
+  };
+
+  // prologue: X(0), X(1) by direct loads, Y(0), Y(1) through registers
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+    if (s < nk) {
+#pragma unroll
+      for (int i = 0; i < XL; ++i) issue_one(s, i);
+      yl.template fetch<0>(s);
+      yl.template commit<0>(lds + s * T::STAGE + T::XBYTES);
+    }
+  UNIT_WAIT_VMCNT(0);
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int i = 0; i < NF; ++i) load_one(lds, 0, 0, i);
+
+  int kt = 0;
+  for (; kt + 2 < nk; ++kt) stage(kt, yes{}, yes{});
+  for (; kt + 1 < nk; ++kt) stage(kt, no{}, yes{});
+  if (kt < nk) stage(kt, no{}, no{});
+
+  Epi::template store<T>(ep, acc, wsx, wsy, x0 + wx * (T::TX * 32), y0 + wy * (T::TY * 32), lane, wave, lds, false);
+}
+
+}  // namespace unit
