@@ -274,6 +274,24 @@ def test_conv3d_c4_every_direct_variant(dev, oracle, monkeypatch):
     assert len(names) >= 15 and all(n.startswith("s8direct_c4") for n in names), names
 
 
+def test_conv2d_largest_output(dev, oracle):
+    """An output just below the 2^31-byte limit (100352 pixels x 5344 channels x 4 bytes = 2.145 GB): 32-bit
+    offsets in the write-back must not wrap.  Checked plane by plane against the oracle run on slices of the
+    weight (first, middle and last 16-channel blocks)."""
+    N, C, H, W, K = 32, 16, 56, 56, 5344
+    assert N * H * W * K * 4 < 2 ** 31 <= N * H * W * (K + 16) * 4
+    data = rng.uniform_u8((N, 1, H, W, 16), 81)
+    wt = rng.uniform_s8((K // 16, 1, 1, 1, 4, 16, 4), 82)
+    out = U.conv2d_NCHWc_int8(_t(data, dev), _t(wt, dev), 1, 0)
+    torch.cuda.synchronize()
+    name = U.last_variant()
+    for ko in (0, 1, K // 32, K // 16 - 2, K // 16 - 1):
+        ref = oracle.c_conv2d_nchwc(data, wt[ko:ko + 1], 1, 0, 1)
+        assert np.array_equal(out[:, ko:ko + 1].cpu().numpy(), ref), (ko, name)
+    del out
+    torch.cuda.empty_cache()
+
+
 def test_conv2d_zero_padding_value(dev, oracle):
     """Padded pixels are u8 zeros: with all-255 data and all-ones weights every output equals
     255 * (number of in-image taps) * C, which differs between border and interior."""
