@@ -357,3 +357,69 @@ def test_conv_chain_through_requantised_activations(dev, oracle):
     out = U.conv2d_NCHWc_int8(mid, U.prepare_conv2d_weight(_t(w2, dev)), 1, 0)
     torch.cuda.synchronize()
     assert np.array_equal(mid.cpu().numpy(), mid_ref) and np.array_equal(out.cpu().numpy(), ref)
+
+
+def _random_conv_cases(count, seed):
+    r = np.random.RandomState(seed)
+    cases = []
+    while len(cases) < count:
+        cb = int(r.choice([4, 16]))
+        cc = int(r.randint(1, 4 if cb == 16 else 3))
+        kh, kw = int(r.randint(1, 6)), int(r.randint(1, 6))
+        sh, sw = int(r.randint(1, 4)), int(r.randint(1, 4))
+        pad = tuple(int(x) for x in r.randint(0, 3, size=4))
+        h, w = int(r.randint(kh, kh + 14)), int(r.randint(kw, kw + 14))
+        dh = int(r.randint(1, 3))
+        if (kh - 1) * dh + 1 > h + pad[0] + pad[2]:
+            continue
+        cases.append((int(r.randint(1, 4)), cc * cb, h, w, 16 * int(r.randint(1, 8)), (kh, kw), (sh, sw), pad, (dh, 1)))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_conv_cases(40, 20240521), ids=lambda c: "x".join(str(v) for v in c[:5]))
+def test_conv2d_random_shapes_all_forms(dev, oracle, case):
+    """Seeded random small configurations (ragged everything: pads, strides, windows, channel counts) through the
+    plain, prepared, fused and requantised entry points."""
+    N, C, H, W, K, (kh, kw), stride, pad, dil = case
+    cb = 16 if C % 16 == 0 else 4
+    seed = N + 3 * C + 5 * H + 7 * W + 11 * K + 13 * kh + 17 * kw
+    data = rng.uniform_u8((N, C // cb, H, W, cb), seed)
+    wt = rng.uniform_s8((K // 16, C // cb, kh, kw, cb // 4, 16, 4), seed + 1)
+    bias = rng.uniform_s8((K,), seed + 2).astype(np.int32) * 997
+    ref = oracle.c_conv2d_nchwc(data, wt, stride, pad, dil)
+    d, w, tb = _t(data, dev), _t(wt, dev), _t(bias, dev)
+    layout = f"NCHW{cb}c"
+    out = U.conv2d_NCHWc_int8(d, w, stride, pad, dil, "int32", layout)
+    assert np.array_equal(out.cpu().numpy(), ref), ("plain", U.last_variant())
+    p = U.prepare_conv2d_weight(w)
+    out = U.conv2d_NCHWc_int8(d, p, stride, pad, dil, "int32", layout)
+    assert np.array_equal(out.cpu().numpy(), ref), ("prepared", U.last_variant())
+    xs = (data ^ 0x80).view(np.int8)
+    ref_f = oracle.conv2d_nchwc_int8_fused(xs, wt, bias, 3, stride, pad, dil, conv=oracle.c_conv2d_nchwc)
+    for kern in (w, p):
+        out = U.conv2d_NCHWc_int8_fused(_t(xs, dev), kern, tb, 3, stride, pad, dil, "int32", layout)
+        assert np.array_equal(out.cpu().numpy(), ref_f), ("fused", U.last_variant())
+    ref_q = oracle.conv2d_nchwc_u8_requant(data, wt, bias, 5, 11, stride, pad, dil, conv=oracle.c_conv2d_nchwc)
+    out = U.conv2d_NCHWc_int8_requant(d, p, tb, 5, 11, stride, pad, dil)
+    assert np.array_equal(out.cpu().numpy(), ref_q), ("requant", U.last_variant())
+
+
+def _random_fp16_cases(count, seed):
+    r = np.random.RandomState(seed)
+    return [(int(r.randint(1, 4)), 16 * int(r.randint(1, 5)), int(r.randint(5, 20)), int(r.randint(5, 20)),
+             16 * int(r.randint(1, 7)), int(r.randint(1, 5)), int(r.randint(1, 3))) for _ in range(count)]
+
+
+@pytest.mark.parametrize("N,C,H,W,K,ks,stride", _random_fp16_cases(16, 77))
+def test_conv2d_fp16_random_shapes(dev, oracle, N, C, H, W, K, ks, stride):
+    a = rng.normal_f16((N, C // 16, H, W, 16), N + C + H)
+    b = rng.normal_f16((K // 16, C // 16, ks, ks, 16, 16), K + ks, 1.0 / np.sqrt(C * ks * ks))
+    ta, tb = _t(a, dev), _t(b, dev)
+    plain = U.conv2d_NCHW16c_OHWI16o(ta, tb, stride, stride)
+    prep = U.conv2d_NCHW16c_OHWI16o(ta, U.prepare_conv2d_weight(tb), stride, stride)
+    torch.cuda.synchronize()
+    ref = oracle.conv2d_nchw16c_f16(a, b, stride, stride)
+    floor = 1e-3 * np.abs(ref).max()
+    for out in (plain, prep):
+        err = float((np.abs(out.cpu().numpy().astype(np.float64) - ref) / np.maximum(np.abs(ref), floor)).max())
+        assert err <= REL_TOL, (err, U.last_variant())
