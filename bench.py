@@ -408,6 +408,10 @@ def main():
     layout = {}
     us = time_us(lambda: U.pack_nchwc(x8, 16), 20)
     layout["pack_nchw16c_u8_32x256x56x56"] = dict(us=round(us, 2), gbs=round(2 * x8.numel() / us / 1e3, 1))
+    p8 = U.pack_nchwc(x8, 16)
+    us = time_us(lambda: U.unpack_nchwc(p8), 20)
+    layout["unpack_nchw16c_u8_32x256x56x56"] = dict(us=round(us, 2), gbs=round(2 * x8.numel() / us / 1e3, 1))
+    del p8
     us = time_us(lambda: U.unpack_nchwc(o32), 20)
     layout["unpack_nchw16c_i32_32x256x56x56"] = dict(us=round(us, 2), gbs=round(2 * o32.numel() * 4 / us / 1e3, 1))
     us = time_us(lambda: U.prepack_conv_weight(w33, 16), 20)

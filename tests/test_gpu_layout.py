@@ -14,7 +14,10 @@ def _t(a, dev):
 
 
 @pytest.mark.parametrize("shape,cb", [((2, 64, 14, 14), 16), ((1, 3, 224, 224), 4), ((1, 35, 7, 9), 16),
-                                      ((3, 10, 5, 5), 4), ((32, 256, 56, 56), 16)])
+                                      ((3, 10, 5, 5), 4), ((32, 256, 56, 56), 16),
+                                      ((2, 40, 8, 8), 16),     # 16-pixel groups, channel tail in the last block
+                                      ((1, 16, 4, 4), 16),     # one 16-pixel group
+                                      ((3, 100, 12, 20), 16)])
 def test_pack_unpack_u8(dev, oracle, shape, cb):
     x = rng.uniform_u8(shape, 1)
     p = U.pack_nchwc(_t(x, dev), cb)

@@ -64,6 +64,81 @@ __global__ __launch_bounds__(256) void nchwc_words(const char *src, char *dst, i
   }
 }
 
+// u8 / s8 with 16-channel blocks and H * W a multiple of 16: a thread moves 16 pixels x 16 channels,
+// 16-byte loads and stores on both sides (16 consecutive pixels of one channel plane <-> one
+// pixel's 16 channels) and a 16 x 16 byte transpose in registers: sixteen 4 x 4 transposes of
+// two v_perm_b32 stages each.  Packing then passes the rows through a wave-private LDS area so that
+// a store instruction writes 64 consecutive pixels (1 KiB) instead of 16-byte pieces 256 bytes
+// apart; LDS operations of one wave execute in order, so the area needs no barrier.
+// 4 x 4 byte transpose: rows a, b, c, d (byte k of a row = column k) -> t[k] = {a.k, b.k, c.k, d.k}
+__device__ __forceinline__ void transpose4x4(u32 a, u32 b, u32 c, u32 d, u32 (&t)[4]) {
+  const u32 x0 = __builtin_amdgcn_perm(b, a, 0x05010400u), x1 = __builtin_amdgcn_perm(b, a, 0x07030602u);
+  const u32 y0 = __builtin_amdgcn_perm(d, c, 0x05010400u), y1 = __builtin_amdgcn_perm(d, c, 0x07030602u);
+  t[0] = __builtin_amdgcn_perm(y0, x0, 0x05040100u);
+  t[1] = __builtin_amdgcn_perm(y0, x0, 0x07060302u);
+  t[2] = __builtin_amdgcn_perm(y1, x1, 0x05040100u);
+  t[3] = __builtin_amdgcn_perm(y1, x1, 0x07060302u);
+}
+
+template <bool PACK>
+__global__ __launch_bounds__(256) void nchw16c_bytes(const char *src, char *dst, int C, int HW, int cc,
+                                                     int groups /* HW / 16 */) {
+  const int g = blockIdx.x * 256 + threadIdx.x;
+  if (!PACK && g >= groups) return;
+  const bool live = g < groups;  // packing: lanes past the end still take part in the wave's write-back
+  const int plane = blockIdx.y;  // n * cc + ci
+  const int n = plane / cc, ci = plane - n * cc;
+  const size_t p0 = (size_t)g * 16;
+  const char *nchw = PACK ? src : dst;
+  const size_t chan0 = ((size_t)n * C + ci * 16) * HW + p0;   // byte offset of channel ci * 16, pixel p0
+  char *blocked = (PACK ? dst : const_cast<char *>(src)) + ((size_t)plane * HW + p0) * 16;
+  v4i planes[16];  // [channel]: 16 pixels
+  v4i rows[16];    // [pixel]: 16 channels
+  if (PACK) {
+#pragma unroll
+    for (int c = 0; c < 16; ++c)
+      planes[c] = live && ci * 16 + c < C ? *reinterpret_cast<const v4i *>(nchw + chan0 + (size_t)c * HW) : v4i{0, 0, 0, 0};
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        u32 t[4];
+        transpose4x4(planes[4 * j][q], planes[4 * j + 1][q], planes[4 * j + 2][q], planes[4 * j + 3][q], t);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) rows[4 * q + k][j] = (int)t[k];
+      }
+    // lane l owns pixels 16 l .. 16 l + 15 of the wave's 1024; pitch 272 bytes per lane: conflict-free both ways
+    __shared__ __attribute__((aligned(16))) char stage[4][64 * 272];
+    const int lane = threadIdx.x & 63;
+    char *st = stage[threadIdx.x >> 6];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) *reinterpret_cast<v4i *>(st + lane * 272 + r * 16) = rows[r];
+    const size_t wave_p0 = p0 - (size_t)lane * 16;  // first pixel of the wave
+    char *out = dst + ((size_t)plane * HW + wave_p0) * 16;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      const int pix = k * 64 + lane;
+      const v4i v = *reinterpret_cast<const v4i *>(st + (pix >> 4) * 272 + (pix & 15) * 16);
+      if (wave_p0 + pix < (size_t)HW) reinterpret_cast<v4i *>(out)[pix] = v;
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) rows[r] = reinterpret_cast<const v4i *>(blocked)[r];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        u32 t[4];
+        transpose4x4(rows[4 * q][j], rows[4 * q + 1][j], rows[4 * q + 2][j], rows[4 * q + 3][j], t);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) planes[4 * j + k][q] = (int)t[k];
+      }
+#pragma unroll
+    for (int c = 0; c < 16; ++c)
+      if (ci * 16 + c < C) *reinterpret_cast<v4i *>(dst + chan0 + (size_t)c * HW) = planes[c];
+  }
+}
+
 // any shape / element size: one thread per blocked element
 template <bool PACK>
 __global__ __launch_bounds__(256) void nchwc_elems(const char *src, char *dst, int C, int HW, int cc, int cb,
@@ -99,7 +174,11 @@ int nchwc(const void *src, void *dst, int N, int C, int H, int W, int cb, int es
   char *out = static_cast<char *>(dst);
   const int HW = (int)hw, pp = 4 / es;
   const bool words = HW % pp == 0 && (cb == 16 || (cb == 4 && es == 1)) && (size_t)N * cc <= 65535;
-  if (words) {
+  if (words && es == 1 && cb == 16 && HW % 16 == 0) {
+    const int groups = HW / 16;
+    hipLaunchKernelGGL(nchw16c_bytes<PACK>, dim3(ceil_div(groups, 256), N * cc), dim3(256), 0, s, in, out, C, HW, cc,
+                       groups);
+  } else if (words) {
     const int groups = HW / pp;
     dim3 grid(ceil_div(groups, 256), N * cc);
 #define UNIT_NCHWC(ES, CB)                                                                                   \
