@@ -130,20 +130,19 @@ __device__ __forceinline__ void store_block_q8(const typename ConvEpilogue<Op>::
     const int rhi = 1 << (p.shift - 33), sh = p.shift - 32;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      u32 packed = 0;
+      int t[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         int v = acc[4 * q + e];
         if (wsb) v += wsb[8 * q + 4 * half + e];
-        int t = min(max((__mulhi(v, p.scale) + rhi) >> sh, 0), 255);
-        // Opaque to the optimiser on purpose: left visible, shift + clamp + pack of two values is
-        // matched to v_ashr_pk_u8_i32, whose result this compiler treats as zero-extended while
-        // the upper 16 bits of the destination came back non-zero (bytes 2 and 3 of the packed
-        // dword read 255 whenever the first value was negative before the shift).
-        asm volatile("" : "+v"(t));
-        packed |= (u32)t << (8 * e);
+        t[e] = __mulhi(v, p.scale) + rhi;
       }
-      d[q] = (int)packed;
+      // v_ashr_pk_u8_i32: shift, saturate to 0..255 and pack two values into the low 16 bits (the
+      // builtin's result is 16 bits wide; the upper half of the register is not zero, and the
+      // byte select below never looks at it)
+      const u32 lo = (unsigned short)__builtin_amdgcn_ashr_pk_u8_i32(t[0], t[1], sh);
+      const u32 hi = (unsigned short)__builtin_amdgcn_ashr_pk_u8_i32(t[2], t[3], sh);
+      d[q] = (int)__builtin_amdgcn_perm(hi, lo, 0x05040100u);
     }
   } else {
     const long long rnd = 1ll << (p.shift - 1);
