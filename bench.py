@@ -350,6 +350,62 @@ def main():
                                "reference's graphs",
                       stack_us=round(rq_us, 1), tops=round(rq_ops / rq_us / 1e6, 2), layers=rq_rows)
 
+    # The Relay-level graph of apps/cpu/relay/conv2d.py:15-27, NCHW int8 in -> NCHW int32 out, as it runs per call
+    # (result.log:30-36): Op #0 data layout transform, Op #5 fused convolution, Op #6 output layout transform --
+    # folded into the convolution's store, and as a kernel of its own.  Weight-side ops #1-#4 are constants.
+    def relay_leg(shapes, batch, iters):
+        rows, tot_f, tot_u, same = [], 0.0, 0.0, True
+        for i, (s, n) in enumerate(shapes):
+            cb = WL.channel_block(s.C)
+            cp = -(-s.C // cb) * cb
+            oh, ow = WL.out_hw(s)
+            x = torch.randint(-128, 128, (n, s.C, s.H, s.W), dtype=torch.int8, device=dev)
+            wt = torch.randint(-128, 128, (s.K, s.C, s.KH, s.KW), dtype=torch.int8, device=dev)
+            bias = dev_t(rng.uniform_s8((s.K,), 6000 + i).astype(np.int32) * 1000)
+            wp = U.prepare_conv2d_weight(U.prepack_conv_weight(wt, cb)).buf
+            data = torch.empty((n, cp // cb, s.H, s.W, cb), dtype=torch.int8, device=dev)
+            o5 = torch.empty((n, s.K // 16, oh, ow, 16), dtype=torch.int32, device=dev)
+            o4 = torch.empty((n, s.K, oh, ow), dtype=torch.int32, device=dev)
+            desc = _lib.ConvDesc(n, cp, s.H, s.W, s.K, s.KH, s.KW, s.stride, s.stride, s.pad, s.pad, s.pad, s.pad, 1, 1, cb)
+
+            def op0():
+                _lib.check(L.unit_pack_nchwc(x.data_ptr(), data.data_ptr(), n, s.C, s.H, s.W, cb, 1, stream))
+
+            def folded():
+                op0()
+                _lib.check(L.unit_conv2d_nchwc_s8s8s32_fused_prepared_nchw(
+                    ctypes.byref(desc), data.data_ptr(), wp.data_ptr(), bias.data_ptr(), 11, o4.data_ptr(), s.K, stream))
+
+            def unfolded():
+                op0()
+                _lib.check(L.unit_conv2d_nchwc_s8s8s32_fused_prepared(
+                    ctypes.byref(desc), data.data_ptr(), wp.data_ptr(), bias.data_ptr(), 11, o5.data_ptr(), stream))
+                _lib.check(L.unit_unpack_nchwc(o5.data_ptr(), o4.data_ptr(), n, s.K, oh, ow, 16, 4, stream))
+
+            unfolded()
+            torch.cuda.synchronize()
+            want = o4.clone()
+            o4.zero_()
+            us_f = time_us(folded, iters)
+            kern = U.last_variant()
+            same = same and torch.equal(o4, want)
+            us_u = time_us(unfolded, iters)
+            rows.append(dict(layer=s.name, batch=n, graph_us=round(us_f, 2), unfolded_us=round(us_u, 2), kernel=kern))
+            tot_f += us_f * s.count
+            tot_u += us_u * s.count
+        return rows, tot_f, tot_u, same
+
+    logged = WL.ConvShape("1x1_1024_2048@16", 1024, 16, 16, 2048, 1, 1, 1, 0, 1)
+    rl_rows, _, _, rl_same0 = relay_leg(((logged, 1),), 1, 30)
+    rl_rows[0].update(reference_us=234.7, reference_source="sum of the seven operators at apps/cpu/relay/result.log:30-36 "
+                                                         "(x86 VNNI, -mcpu=cascadelake; 206.0 us without the weight-side operators #1-#4)")
+    r50_rows, r50_f, r50_u, rl_same = relay_leg(tuple((s, BATCH) for s in WL.RESNET50), BATCH, 20)
+    relay_graph = dict(workload="(conv2d(x, w) + b) * 11, x int8 NCHW -> int32 NCHW (apps/cpu/relay/conv2d.py:15-27): data layout "
+                                "transform + fused convolution storing NCHW; `unfolded` runs the output layout transform as its own kernel",
+                       logged_graph=rl_rows[0], resnet50_b32_stack_us=round(r50_f, 1),
+                       resnet50_b32_unfolded_stack_us=round(r50_u, 1), folded_equals_unfolded=bool(rl_same and rl_same0),
+                       layers=r50_rows)
+
     # 3-D convolution workloads of apps/cpu/kernel/conv3d.py:13-25 (depth 16, batch 1)
     c3_rows = []
     for i, (ic, h, w_, oc, ks, st) in enumerate(((256, 16, 16, 256, 3, 1), (512, 9, 9, 512, 3, 1), (128, 30, 30, 128, 3, 1),
@@ -514,6 +570,7 @@ def main():
         "conv_fp16_resnet50_b32": conv_fp16,
         "conv_fused_s8_resnet50_b32": fused_s8,
         "conv_requant_u8_resnet50_b32": requant_u8,
+        "relay_graph_s8": relay_graph,
         "conv3d_s8": conv3d,
         "layout_kernels": layout,
         "layers": table,

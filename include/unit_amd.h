@@ -223,6 +223,14 @@ int unit_conv2d_nchwc_s8s8s32_fused_prepared(const unit_conv_desc *d, const void
 int unit_conv2d_nchw16c_f16f32_prepared(const unit_conv_desc *d, const void *a, const void *prepared,
                                         void *out, unit_stream_t stream);
 
+/* unit_conv2d_nchwc_s8s8s32_fused_prepared with the graph's closing layout_transform NCHW16c -> NCHW
+ * (apps/cpu/relay/result.log:25, Op "fused_layout_transform" of :36) folded into the store:
+ * out is (N, out_channels, OH, OW) int32, d->K - 16 < out_channels <= d->K (channels the caller
+ * padded up to a multiple of 16 are not written). */
+int unit_conv2d_nchwc_s8s8s32_fused_prepared_nchw(const unit_conv_desc *d, const void *data, const void *prepared,
+                                                  const int32_t *bias, int32_t scale, void *out,
+                                                  int32_t out_channels, unit_stream_t stream);
+
 /* u8 x s8 convolution on prepared weights with the output requantised to u8 in the blocked
  * layout the next convolution reads, (N, K/16, OH, OW, 16) u8:
  *   q = clamp(((conv_u8(data, w)[k] + bias[k]) * scale + 2^(shift-1)) >> shift, 0, 255)

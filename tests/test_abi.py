@@ -102,6 +102,14 @@ def test_out_hw_and_error_paths_without_gpu():
     assert L.unit_conv2d_nchwc_s8s8s32_fused_prepared(ctypes.byref(big), 1, 1, None, 1, 1, None) == -1 and b"31 positions" in L.unit_last_error()
     pad = _lib.ConvDesc(1, 16, 20, 20, 16, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 16)
     assert L.unit_conv2d_nchw16c_f16f32_prepared(ctypes.byref(pad), 1, 1, 1, None) == -1 and b"padding" in L.unit_last_error()
+    # NCHW output: the channel count must round up to K
+    ok32 = _lib.ConvDesc(1, 16, 8, 8, 32, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 16)
+    for oc in (16, 33, 0, -1):
+        assert L.unit_conv2d_nchwc_s8s8s32_fused_prepared_nchw(ctypes.byref(ok32), 16, 16, None, 1, 16, oc, None) == -1
+        assert b"does not round up" in L.unit_last_error()
+    assert L.unit_conv2d_nchwc_s8s8s32_fused_prepared_nchw(ctypes.byref(ok32), 16, 16, None, 1, 8, 17, None) == -1
+    assert b"aligned" in L.unit_last_error()
+    assert L.unit_conv2d_nchwc_s8s8s32_fused_prepared_nchw(None, 16, 16, None, 1, 16, 17, None) == -1 and b"null" in L.unit_last_error()
     # tensor pointers must be 16-byte aligned (the kernels use 16-byte vector accesses)
     ok = _lib.ConvDesc(1, 16, 8, 8, 16, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 16)
     for args in ((8, 16, 16), (16, 4, 16), (16, 16, 24)):

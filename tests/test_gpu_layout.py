@@ -17,7 +17,14 @@ def _t(a, dev):
                                       ((3, 10, 5, 5), 4), ((32, 256, 56, 56), 16),
                                       ((2, 40, 8, 8), 16),     # 16-pixel groups, channel tail in the last block
                                       ((1, 16, 4, 4), 16),     # one 16-pixel group
-                                      ((3, 100, 12, 20), 16)])
+                                      ((3, 100, 12, 20), 16),
+                                      ((32, 512, 7, 7), 16),    # 49-pixel planes: three full groups and one pixel
+                                      ((5, 33, 7, 7), 16),      # ... with a channel tail
+                                      ((2, 64, 17, 17), 16),    # odd plane size, unaligned plane starts
+                                      ((3, 20, 3, 5), 16),      # planes smaller than a group
+                                      ((1, 16, 1, 1), 16),
+                                      ((1, 2000, 5, 6), 16),    # many planes, groups of 16 + 14
+                                      ((32, 128, 28, 28), 16)])
 def test_pack_unpack_u8(dev, oracle, shape, cb):
     x = rng.uniform_u8(shape, 1)
     p = U.pack_nchwc(_t(x, dev), cb)

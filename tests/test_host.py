@@ -68,3 +68,11 @@ def test_rng_streams():
     assert abs(z.mean()) < 0.02 and abs(z.std() - 1.0) < 0.02
     assert np.array_equal(rng.uniform_u8((100,), 5), rng.uniform_u8((100,), 5))
     assert not np.array_equal(rng.uniform_u8((100,), 5), rng.uniform_u8((100,), 6))
+
+
+def test_relay_driver_wants_ten_integers():
+    from unit_amd import relay
+    with pytest.raises(SystemExit, match="usage"):
+        relay.main(["1", "2", "3"])
+    with pytest.raises(SystemExit, match="differ"):
+        relay.main("1 32 14 14 32 16 3 3 1 1".split())

@@ -35,6 +35,7 @@ SYMBOLS = (
     "unit_conv2d_prepare_weight",
     "unit_conv2d_nchwc_u8s8s32_prepared",
     "unit_conv2d_nchwc_s8s8s32_fused_prepared",
+    "unit_conv2d_nchwc_s8s8s32_fused_prepared_nchw",
     "unit_conv2d_nchw16c_f16f32_prepared",
     "unit_conv2d_nchwc_u8s8u8_requant_prepared",
     "unit_mfma_tile_i8",
@@ -96,6 +97,7 @@ def load():
     L.unit_conv2d_prepare_weight.argtypes = [i32, i32, i32, i32, i32, i32, vp, vp, vp]
     L.unit_conv2d_nchwc_u8s8s32_prepared.argtypes = [dp, vp, vp, vp, vp]
     L.unit_conv2d_nchwc_s8s8s32_fused_prepared.argtypes = [dp, vp, vp, vp, i32, vp, vp]
+    L.unit_conv2d_nchwc_s8s8s32_fused_prepared_nchw.argtypes = [dp, vp, vp, vp, i32, vp, i32, vp]
     L.unit_conv2d_nchw16c_f16f32_prepared.argtypes = [dp, vp, vp, vp, vp]
     L.unit_conv2d_nchwc_u8s8u8_requant_prepared.argtypes = [dp, vp, vp, vp, i32, i32, vp, vp]
     L.unit_mfma_tile_i8.argtypes = [vp, vp, vp, vp]

@@ -84,6 +84,27 @@ __device__ __forceinline__ void store_block(const typename ConvEpilogue<Op>::Par
   constexpr int kPitch = 144;
   const int l32 = lane & 31, half = lane >> 5;
   const int rp = lane >> 2, piece = lane & 3;
+  if (p.planar) {
+    // (N, planar, OH, OW): register r of a lane is channel 8 (r / 4) + 4 half + r % 4 of the lane's pixel, so
+    // a register of 32 lanes is 128 consecutive bytes of one channel plane: no transpose
+    const int m = m0 + l32;
+    int n, pix;
+    p.by_ohw.divmod(m, n, pix);
+    out_t *dst = reinterpret_cast<out_t *>(p.out) + ((size_t)n * p.planar + c0 + 4 * half) * p.ohw + pix;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      out4_t v = {acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]};
+      if constexpr (Op::kInt) {
+        if (wsb) v += *reinterpret_cast<const v4i *>(wsb + 8 * q + 4 * half);
+        if (scale != 1) v *= scale;
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (c0 + 8 * q + 4 * half + e < p.planar && m < p.npix)
+          __builtin_nontemporal_store(v[e], dst + (size_t)(8 * q + e) * p.ohw);
+    }
+    return;
+  }
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     out4_t v = {acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]};

@@ -8,7 +8,7 @@ namespace unit {
 template <class Op, class S, bool SHIFT, bool PREP = false, bool C4 = false, bool Q8 = false>
 int run_direct(const char *what, const char *tag, const unit_conv_desc *d, const ConvGeom &g, const void *data,
                const void *w, const int *bias, int scale, void *out, const ConvPlan &plan, hipStream_t s,
-               const int *bias2 = nullptr, int shift = 0) {
+               const int *bias2 = nullptr, int shift = 0, int planar = 0) {
   const int ntab = C4 ? 2 * g.c4_steps : (Op::kInt ? 2 * ((g.ntaps + 1) / 2) : g.ntaps);
   const int lds = S::template lds_fixed<Op>() + ntab * 8;
   if (lds > kMaxLds) return fail(UNIT_E_ARG, "%s: needs %d bytes of LDS (limit %d)", what, lds, kMaxLds);
@@ -20,7 +20,7 @@ int run_direct(const char *what, const char *tag, const unit_conv_desc *d, const
     if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "%s: hipFuncSetAttribute: %s", what, hipGetErrorString(e));
     lds_allowed = kMaxLds;
   }
-  typename ConvEpilogue<Op>::Params ep{out, d->K, g.by_ohw.d, g.npix, g.by_ohw, bias, scale, bias2, shift};
+  typename ConvEpilogue<Op>::Params ep{out, d->K, g.by_ohw.d, g.npix, g.by_ohw, bias, scale, bias2, shift, planar};
   GridMap gm;
   gm.gx = ceil_div(d->K, S::BX);
   gm.gy = ceil_div(g.npix, S::BY);

@@ -14,9 +14,9 @@ const TunedConv *tuned_conv_i8_prepared(int *n);                                
 int conv_u8_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
                      const int *addend, void *out, hipStream_t s);  // conv_prepared_u8.hip
 int conv_s8_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
-                     const int *bias, int scale, void *out, hipStream_t s);  // conv_prepared_s8.hip
+                     const int *bias, int scale, void *out, int planar, hipStream_t s);  // conv_prepared_s8.hip
 int conv_c4_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
-                     const int *addend, int scale, bool shift, void *out, hipStream_t s);  // conv_prepared_c4.hip
+                     const int *addend, int scale, bool shift, void *out, int planar, hipStream_t s);  // conv_prepared_c4.hip
 int conv_q8_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
                      const int *addend, const int *bias, int scale, int shift, void *out, hipStream_t s);  // conv_prepared_q8.hip
 int conv_f16_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *a, const void *w,
@@ -194,7 +194,7 @@ extern "C" int unit_conv2d_nchwc_u8s8s32_prepared(const unit_conv_desc *d, const
   const char *w = static_cast<const char *>(prepared);
   const int *addend = reinterpret_cast<const int *>(w + pl.frag_bytes);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (d->cb == 4) return conv_c4_prepared(p, d, g, data, w, addend, 1, true, out, s);
+  if (d->cb == 4) return conv_c4_prepared(p, d, g, data, w, addend, 1, true, out, 0, s);
   return conv_u8_prepared(p, d, g, data, w, addend, out, s);
 }
 
@@ -221,19 +221,39 @@ extern "C" int unit_conv2d_nchwc_u8s8u8_requant_prepared(const unit_conv_desc *d
                           static_cast<hipStream_t>(stream));
 }
 
-extern "C" int unit_conv2d_nchwc_s8s8s32_fused_prepared(const unit_conv_desc *d, const void *data,
-                                                        const void *prepared, const int32_t *bias, int32_t scale,
-                                                        void *out, unit_stream_t stream) {
-  using namespace unit;
-  const char *what = "unit_conv2d_nchwc_s8s8s32_fused_prepared";
+namespace unit {
+namespace {
+
+// planar: 0 = blocked output, else the channel count of the (N, planar, OH, OW) output
+int fused_prepared(const char *what, const unit_conv_desc *d, const void *data, const void *prepared,
+                   const int32_t *bias, int32_t scale, void *out, int planar, unit_stream_t stream) {
   if (!d || !data || !prepared || !out) return fail(UNIT_E_ARG, "%s: null pointer", what);
   ConvGeom g;
   if (int rc = check_prepared_conv(what, d, 16, &g, data, prepared, out)) return rc;
   const int ntable = (int)(sizeof(kTunedI8Prepared) / sizeof(kTunedI8Prepared[0])) - 1;
   const ConvPlan p = plan_prepared(d, g, g.ntaps * d->cb, kTunedI8Prepared, ntable, true);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (d->cb == 4) return conv_c4_prepared(p, d, g, data, prepared, bias, scale, false, out, s);
-  return conv_s8_prepared(p, d, g, data, prepared, bias, scale, out, s);
+  if (d->cb == 4) return conv_c4_prepared(p, d, g, data, prepared, bias, scale, false, out, planar, s);
+  return conv_s8_prepared(p, d, g, data, prepared, bias, scale, out, planar, s);
+}
+
+}  // namespace
+}  // namespace unit
+
+extern "C" int unit_conv2d_nchwc_s8s8s32_fused_prepared(const unit_conv_desc *d, const void *data,
+                                                        const void *prepared, const int32_t *bias, int32_t scale,
+                                                        void *out, unit_stream_t stream) {
+  return unit::fused_prepared("unit_conv2d_nchwc_s8s8s32_fused_prepared", d, data, prepared, bias, scale, out, 0, stream);
+}
+
+extern "C" int unit_conv2d_nchwc_s8s8s32_fused_prepared_nchw(const unit_conv_desc *d, const void *data,
+                                                             const void *prepared, const int32_t *bias, int32_t scale,
+                                                             void *out, int32_t out_channels, unit_stream_t stream) {
+  using namespace unit;
+  const char *what = "unit_conv2d_nchwc_s8s8s32_fused_prepared_nchw";
+  if (d && (out_channels <= d->K - 16 || out_channels > d->K))
+    return fail(UNIT_E_ARG, "%s: out_channels %d does not round up to K = %d", what, out_channels, d->K);
+  return fused_prepared(what, d, data, prepared, bias, scale, out, out_channels, stream);
 }
 
 extern "C" int unit_conv2d_nchw16c_f16f32_prepared(const unit_conv_desc *d, const void *a, const void *prepared,

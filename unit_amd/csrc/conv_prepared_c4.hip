@@ -5,15 +5,18 @@
 namespace unit {
 
 int conv_c4_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
-                     const int *addend, int scale, bool shift, void *out, hipStream_t s) {
-  const char *what = shift ? "unit_conv2d_nchwc_u8s8s32_prepared" : "unit_conv2d_nchwc_s8s8s32_fused_prepared";
+                     const int *addend, int scale, bool shift, void *out, int planar, hipStream_t s) {
+  const char *what = shift    ? "unit_conv2d_nchwc_u8s8s32_prepared"
+                     : planar ? "unit_conv2d_nchwc_s8s8s32_fused_prepared_nchw"
+                              : "unit_conv2d_nchwc_s8s8s32_fused_prepared";
+  const char *tag = planar ? "s8prep_c4_nchw" : "s8prep_c4";
 #define UNIT_CONV_VARIANT(ID, BX, BY, BKB, WX, WY, PF, FF, KG)
 #define UNIT_CONV_DIRECT(ID, TX, TY, KG, D)                                                                            \
   case ID:                                                                                                             \
     return shift ? run_direct<OpI8, DirectShape<TX, TY, KG, D, true>, true, true, true>(what, "i8prep_c4", d, g, data, \
                                                                                          w, addend, 1, out, plan, s)   \
                  : run_direct<OpI8, DirectShape<TX, TY, KG, D, true>, false, true, true>(                              \
-                       what, "s8prep_c4", d, g, data, w, addend, scale, out, plan, s);
+                       what, tag, d, g, data, w, addend, scale, out, plan, s, nullptr, 0, planar);
   switch (plan.variant) {
 #include "conv_variants.def"
     default:

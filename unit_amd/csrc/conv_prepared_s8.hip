@@ -5,16 +5,17 @@
 namespace unit {
 
 int conv_s8_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
-                     const int *bias, int scale, void *out, hipStream_t s) {
-  const char *what = "unit_conv2d_nchwc_s8s8s32_fused_prepared";
+                     const int *bias, int scale, void *out, int planar, hipStream_t s) {
+  const char *what = planar ? "unit_conv2d_nchwc_s8s8s32_fused_prepared_nchw" : "unit_conv2d_nchwc_s8s8s32_fused_prepared";
+  const char *tag = planar ? "s8prep_c16_nchw" : "s8prep_c16";
   const bool masked = d->pt || d->pl || d->pb || d->pr;
 #define UNIT_CONV_VARIANT(ID, BX, BY, BKB, WX, WY, PF, FF, KG)
 #define UNIT_CONV_DIRECT(ID, TX, TY, KG, D)                                                                             \
   case ID:                                                                                                              \
-    return masked ? run_direct<OpI8, DirectShape<TX, TY, KG, D, true>, false, true>(what, "s8prep_c16", d, g, data, w,  \
-                                                                                     bias, scale, out, plan, s)         \
-                  : run_direct<OpI8, DirectShape<TX, TY, KG, D, false>, false, true>(what, "s8prep_c16", d, g, data, w, \
-                                                                                      bias, scale, out, plan, s);
+    return masked ? run_direct<OpI8, DirectShape<TX, TY, KG, D, true>, false, true>(                                    \
+                        what, tag, d, g, data, w, bias, scale, out, plan, s, nullptr, 0, planar)                        \
+                  : run_direct<OpI8, DirectShape<TX, TY, KG, D, false>, false, true>(                                   \
+                        what, tag, d, g, data, w, bias, scale, out, plan, s, nullptr, 0, planar);
   switch (plan.variant) {
 #include "conv_variants.def"
     default:

@@ -77,6 +77,9 @@ struct ConvEpilogue {
     // requantised u8 output (direct kernels, Q8): a second per-channel addend and the right shift
     const int *bias2;
     int shift;
+    // direct kernels: 0 = blocked (N, K/16, OH, OW, 16) output; else the output is planar (N, planar, OH, OW),
+    // planar <= K channels (the reference's graphs end in this layout_transform: apps/cpu/relay/result.log:25)
+    int planar;
   };
   static constexpr int kPitch = 144;               // bytes per pixel row of the scratch
   static constexpr int kScratch = 32 * kPitch;     // per wave

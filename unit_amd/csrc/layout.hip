@@ -64,12 +64,15 @@ __global__ __launch_bounds__(256) void nchwc_words(const char *src, char *dst, i
   }
 }
 
-// u8 / s8 with 16-channel blocks and H * W a multiple of 16: a thread moves 16 pixels x 16 channels,
-// 16-byte loads and stores on both sides (16 consecutive pixels of one channel plane <-> one
+// u8 / s8 with 16-channel blocks: a thread moves 16 pixels x 16 channels of one (image, channel block)
+// plane, 16-byte loads and stores on both sides (16 consecutive pixels of one channel plane <-> one
 // pixel's 16 channels) and a 16 x 16 byte transpose in registers: sixteen 4 x 4 transposes of
 // two v_perm_b32 stages each.  Packing then passes the rows through a wave-private LDS area so that
 // a store instruction writes 64 consecutive pixels (1 KiB) instead of 16-byte pieces 256 bytes
 // apart; LDS operations of one wave execute in order, so the area needs no barrier.
+// The work items are the 16-pixel groups of all planes in one flat index (small planes still fill
+// the blocks); a plane of fewer than 16 pixels is one partial group that goes byte by byte on the
+// NCHW side.
 // 4 x 4 byte transpose: rows a, b, c, d (byte k of a row = column k) -> t[k] = {a.k, b.k, c.k, d.k}
 __device__ __forceinline__ void transpose4x4(u32 a, u32 b, u32 c, u32 d, u32 (&t)[4]) {
   const u32 x0 = __builtin_amdgcn_perm(b, a, 0x05010400u), x1 = __builtin_amdgcn_perm(b, a, 0x07030602u);
@@ -80,24 +83,41 @@ __device__ __forceinline__ void transpose4x4(u32 a, u32 b, u32 c, u32 d, u32 (&t
   t[3] = __builtin_amdgcn_perm(y1, x1, 0x07060302u);
 }
 
+// 16 bytes at any byte address (a group's first byte in a plane of H * W bytes)
+typedef int bytes16_t __attribute__((ext_vector_type(4), aligned(1)));
+
 template <bool PACK>
 __global__ __launch_bounds__(256) void nchw16c_bytes(const char *src, char *dst, int C, int HW, int cc,
-                                                     int groups /* HW / 16 */) {
-  const int g = blockIdx.x * 256 + threadIdx.x;
-  if (!PACK && g >= groups) return;
-  const bool live = g < groups;  // packing: lanes past the end still take part in the wave's write-back
-  const int plane = blockIdx.y;  // n * cc + ci
+                                                     FastDiv by_groups /* ceil(HW / 16) */, int total_groups) {
+  const int gid = blockIdx.x * 256 + threadIdx.x;
+  if (!PACK && gid >= total_groups) return;
+  const bool live = gid < total_groups;  // packing: lanes past the end still take part in the wave's write-back
+  int plane, g;                          // plane = n * cc + ci
+  by_groups.divmod(live ? gid : 0, plane, g);
   const int n = plane / cc, ci = plane - n * cc;
-  const size_t p0 = (size_t)g * 16;
+  // the last group of a plane is moved back to end with the plane (it overlaps its neighbour, and both
+  // write the same bytes there); only planes of fewer than 16 pixels have a partial group
+  const int p0 = g * 16 + 16 <= HW || HW < 16 ? g * 16 : HW - 16;
+  const int cnt = live ? min(16, HW - p0) : 0;  // pixels of this group
   const char *nchw = PACK ? src : dst;
-  const size_t chan0 = ((size_t)n * C + ci * 16) * HW + p0;   // byte offset of channel ci * 16, pixel p0
-  char *blocked = (PACK ? dst : const_cast<char *>(src)) + ((size_t)plane * HW + p0) * 16;
+  const size_t chan0 = ((size_t)n * C + ci * 16) * HW + p0;  // byte offset of channel ci * 16, pixel p0
+  const size_t flat0 = (size_t)plane * HW + p0;              // pixel index in the blocked tensor
   v4i planes[16];  // [channel]: 16 pixels
   v4i rows[16];    // [pixel]: 16 channels
   if (PACK) {
+    if (cnt == 16) {
 #pragma unroll
-    for (int c = 0; c < 16; ++c)
-      planes[c] = live && ci * 16 + c < C ? *reinterpret_cast<const v4i *>(nchw + chan0 + (size_t)c * HW) : v4i{0, 0, 0, 0};
+      for (int c = 0; c < 16; ++c)
+        planes[c] = ci * 16 + c < C ? (v4i) * reinterpret_cast<const bytes16_t *>(nchw + chan0 + (size_t)c * HW) : v4i{0, 0, 0, 0};
+    } else {
+#pragma unroll
+      for (int c = 0; c < 16; ++c) {
+        u32 w[4] = {0, 0, 0, 0};
+        if (ci * 16 + c < C)
+          for (int e = 0; e < cnt; ++e) w[e >> 2] |= (u32)(unsigned char)nchw[chan0 + (size_t)c * HW + e] << (8 * (e & 3));
+        planes[c] = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+      }
+    }
 #pragma unroll
     for (int q = 0; q < 4; ++q)
 #pragma unroll
@@ -107,23 +127,26 @@ __global__ __launch_bounds__(256) void nchw16c_bytes(const char *src, char *dst,
 #pragma unroll
         for (int k = 0; k < 4; ++k) rows[4 * q + k][j] = (int)t[k];
       }
-    // lane l owns pixels 16 l .. 16 l + 15 of the wave's 1024; pitch 272 bytes per lane: conflict-free both ways
+    // lane l parks its 16 rows at pitch 272 bytes (conflict-free both ways) with the group's first pixel and
+    // pixel count behind them; the wave then stores row after row, 64 rows per instruction
     __shared__ __attribute__((aligned(16))) char stage[4][64 * 272];
     const int lane = threadIdx.x & 63;
     char *st = stage[threadIdx.x >> 6];
 #pragma unroll
     for (int r = 0; r < 16; ++r) *reinterpret_cast<v4i *>(st + lane * 272 + r * 16) = rows[r];
-    const size_t wave_p0 = p0 - (size_t)lane * 16;  // first pixel of the wave
-    char *out = dst + ((size_t)plane * HW + wave_p0) * 16;
+    *reinterpret_cast<v2i *>(st + lane * 272 + 256) = v2i{(int)flat0, cnt};
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
       const int pix = k * 64 + lane;
-      const v4i v = *reinterpret_cast<const v4i *>(st + (pix >> 4) * 272 + (pix & 15) * 16);
-      if (wave_p0 + pix < (size_t)HW) reinterpret_cast<v4i *>(out)[pix] = v;
+      const char *slot = st + (pix >> 4) * 272;
+      const v4i v = *reinterpret_cast<const v4i *>(slot + (pix & 15) * 16);
+      const v2i where = *reinterpret_cast<const v2i *>(slot + 256);
+      if ((pix & 15) < where[1]) reinterpret_cast<v4i *>(dst)[(size_t)where[0] + (pix & 15)] = v;
     }
   } else {
+    const v4i *blocked = reinterpret_cast<const v4i *>(src) + flat0;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) rows[r] = reinterpret_cast<const v4i *>(blocked)[r];
+    for (int r = 0; r < 16; ++r) rows[r] = r < cnt ? blocked[r] : v4i{0, 0, 0, 0};
 #pragma unroll
     for (int q = 0; q < 4; ++q)
 #pragma unroll
@@ -133,9 +156,16 @@ __global__ __launch_bounds__(256) void nchw16c_bytes(const char *src, char *dst,
 #pragma unroll
         for (int k = 0; k < 4; ++k) planes[4 * j + k][q] = (int)t[k];
       }
+    if (cnt == 16) {
 #pragma unroll
-    for (int c = 0; c < 16; ++c)
-      if (ci * 16 + c < C) *reinterpret_cast<v4i *>(dst + chan0 + (size_t)c * HW) = planes[c];
+      for (int c = 0; c < 16; ++c)
+        if (ci * 16 + c < C) *reinterpret_cast<bytes16_t *>(dst + chan0 + (size_t)c * HW) = (bytes16_t)planes[c];
+    } else {
+#pragma unroll
+      for (int c = 0; c < 16; ++c)
+        if (ci * 16 + c < C)
+          for (int e = 0; e < cnt; ++e) dst[chan0 + (size_t)c * HW + e] = (char)((u32)planes[c][e >> 2] >> (8 * (e & 3)));
+    }
   }
 }
 
@@ -174,10 +204,11 @@ int nchwc(const void *src, void *dst, int N, int C, int H, int W, int cb, int es
   char *out = static_cast<char *>(dst);
   const int HW = (int)hw, pp = 4 / es;
   const bool words = HW % pp == 0 && (cb == 16 || (cb == 4 && es == 1)) && (size_t)N * cc <= 65535;
-  if (words && es == 1 && cb == 16 && HW % 16 == 0) {
-    const int groups = HW / 16;
-    hipLaunchKernelGGL(nchw16c_bytes<PACK>, dim3(ceil_div(groups, 256), N * cc), dim3(256), 0, s, in, out, C, HW, cc,
-                       groups);
+  if (es == 1 && cb == 16) {
+    const int groups = ceil_div(HW, 16), total_groups = N * cc * groups;  // < 2^27: the tensor fits 2^31 bytes
+    const dim3 grid(ceil_div(total_groups, 256));
+    const FastDiv by_groups = FastDiv::make(groups);
+    hipLaunchKernelGGL(nchw16c_bytes<PACK>, grid, dim3(256), 0, s, in, out, C, HW, cc, by_groups, total_groups);
   } else if (words) {
     const int groups = HW / pp;
     dim3 grid(ceil_div(groups, 256), N * cc);

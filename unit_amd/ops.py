@@ -195,7 +195,7 @@ def conv2d_NCHWc_int8(data, kernel, stride, padding, dilation=1, out_dtype="int3
 
 
 def conv2d_NCHWc_int8_fused(data, kernel, bias, scale, stride, padding, dilation=1, out_dtype="int32",
-                            layout="NCHW16c", out_layout="NCHW16c"):
+                            layout="NCHW16c", out_layout="NCHW16c", out_channels=None):
     """The quantized model form of the convolution,
     fused_nn_contrib_conv2d_NCHWc_subtract_add_multiply (apps/cpu/relay/result.log:3-26,35):
 
@@ -208,6 +208,10 @@ def conv2d_NCHWc_int8_fused(data, kernel, bias, scale, stride, padding, dilation
     bias   int32 (K,) / any shape with K elements, or None
     scale  Python int
     returns int32 (N, K/16, OH, OW, 16)
+
+    out_layout='NCHW' (prepared weights only) folds the graph's closing layout_transform
+    (result.log:25) into the store: returns int32 (N, out_channels, OH, OW), out_channels
+    (default K) being the channel count before the caller padded it up to a multiple of 16.
     """
     import ctypes
     data = _dev(data, "data", torch.int8, 5)
@@ -217,8 +221,13 @@ def conv2d_NCHWc_int8_fused(data, kernel, bias, scale, stride, padding, dilation
     if out_dtype != "int32":
         raise ValueError(f"out_dtype: only 'int32' is supported, got {out_dtype!r}")
     _layout_block(layout, "layout")
-    if _layout_block(out_layout, "out_layout") != 16:
-        raise ValueError("out_layout: the output channel block is 16 (NCHW16c)")
+    planar = out_layout == "NCHW"
+    if planar and not prepared:
+        raise ValueError("out_layout: 'NCHW' needs prepared weights (prepare_conv2d_weight)")
+    if not planar and out_channels is not None:
+        raise ValueError("out_channels: only with out_layout='NCHW'")
+    if not planar and _layout_block(out_layout, "out_layout") != 16:
+        raise ValueError("out_layout: the output channel block is 16 (NCHW16c), or 'NCHW'")
     n, cc, h, w, cb = data.shape
     if cb not in (4, 16):
         raise ValueError(f"data: channel block must be 16 or 4, got {cb}")
@@ -243,6 +252,15 @@ def conv2d_NCHWc_int8_fused(data, kernel, bias, scale, stride, padding, dilation
     L = _lib.load()
     oh, ow = ctypes.c_int32(), ctypes.c_int32()
     check(L.unit_conv_out_hw(ctypes.byref(d), ctypes.byref(oh), ctypes.byref(ow)))
+    if planar:
+        oc = ko * 16 if out_channels is None else int(out_channels)
+        if not ko * 16 - 16 < oc <= ko * 16:
+            raise ValueError(f"out_channels: {oc} does not round up to K = {ko * 16}")
+        out = torch.empty((n, oc, oh.value, ow.value), dtype=torch.int32, device=data.device)
+        check(L.unit_conv2d_nchwc_s8s8s32_fused_prepared_nchw(
+            ctypes.byref(d), data.data_ptr(), kernel.buf.data_ptr(), bias.data_ptr() if bias is not None else None,
+            scale, out.data_ptr(), oc, _stream()))
+        return out
     out = torch.empty((n, ko, oh.value, ow.value, 16), dtype=torch.int32, device=data.device)
     fn = L.unit_conv2d_nchwc_s8s8s32_fused_prepared if prepared else L.unit_conv2d_nchwc_s8s8s32_fused
     check(fn(ctypes.byref(d), data.data_ptr(), kernel.buf.data_ptr() if prepared else kernel.data_ptr(),
