@@ -350,6 +350,32 @@ def main():
                                "reference's graphs",
                       stack_us=round(rq_us, 1), tops=round(rq_ops / rq_us / 1e6, 2), layers=rq_rows)
 
+    # The same network as a chain: the 52 convolutions behind the stem, each reading the u8 NCHW16c output of the one
+    # before it (projection shortcuts as side branches), buffers owned by the runner, replayed as one HIP graph.
+    from unit_amd import chain as CH
+    ch_layers = CH.resnet50_layers(lambda oc, ic, k: torch.randint(-128, 128, (oc, ic, k, k), dtype=torch.int8, device=dev),
+                                   lambda oc: torch.randint(-1000, 1000, (oc,), dtype=torch.int32, device=dev))
+    ch = CH.ConvChain(ch_layers, (BATCH, 4, 56, 56, 16))
+    ch_x = torch.randint(0, 256, (BATCH, 4, 56, 56, 16), dtype=torch.uint8, device=dev)
+    for i, ly in enumerate(ch_layers):  # per-layer shift from the layer's own int32 sums: activations stay spread over 0..255
+        acc = U.conv2d_NCHWc_int8(ch.source_of(i, ch_x), ch.weights[i], ly.stride, ly.padding)
+        p95 = float(torch.quantile(acc.flatten()[::61][:1 << 20].float(), 0.95))
+        ch.consts[i] = (3, max(1, int(np.ceil(np.log2(max(p95, 1.0) * 3 / 200)))))
+        ch.launch_layer(i, ch_x)
+        del acc
+    ch_alive = min(float((o[:1] > 0).float().mean()) for o in ch.outputs)
+    ch_iso = sum(time_us(lambda i=i: ch.launch_layer(i, ch_x), 20) for i in range(len(ch_layers)))
+    ch_eager = time_us(lambda: ch.run(ch_x), 10)
+    ch_replay = ch.graph(ch_x)
+    ch_graph = time_us(ch_replay, 10)
+    ch_ops = sum(2 * WL.macs(s_, BATCH) * s_.count for s_ in WL.RESNET50[1:])
+    conv_chain = dict(workload="ResNet-50 v1 behind the stem as a chain: 52 requantising convolutions, batch 32, each reading the "
+                               "u8 NCHW16c output of the one before it (projection shortcuts as side branches; residual additions "
+                               "are not part of the path); an extension like the requantised output itself",
+                      hipgraph_us=round(ch_graph, 1), eager_us=round(ch_eager, 1), sum_of_isolated_layers_us=round(ch_iso, 1),
+                      tops=round(ch_ops / ch_graph / 1e6, 2), min_fraction_of_nonzero_activations=round(ch_alive, 3))
+    del ch, ch_replay
+
     # The Relay-level graph of apps/cpu/relay/conv2d.py:15-27, NCHW int8 in -> NCHW int32 out, as it runs per call
     # (result.log:30-36): Op #0 data layout transform, Op #5 fused convolution, Op #6 output layout transform --
     # folded into the convolution's store, and as a kernel of its own.  Weight-side ops #1-#4 are constants.
@@ -570,6 +596,7 @@ def main():
         "conv_fp16_resnet50_b32": conv_fp16,
         "conv_fused_s8_resnet50_b32": fused_s8,
         "conv_requant_u8_resnet50_b32": requant_u8,
+        "conv_chain_u8_resnet50_b32": conv_chain,
         "relay_graph_s8": relay_graph,
         "conv3d_s8": conv3d,
         "layout_kernels": layout,

@@ -76,3 +76,22 @@ def test_relay_driver_wants_ten_integers():
         relay.main(["1", "2", "3"])
     with pytest.raises(SystemExit, match="differ"):
         relay.main("1 32 14 14 32 16 3 3 1 1".split())
+
+
+def test_resnet50_chain_lists_the_logged_shapes():
+    """The chain's 52 layers are exactly the reference's ResNet-50 shape list without the stem, with its multiplicities."""
+    from collections import Counter
+    from unit_amd import chain
+    layers = chain.resnet50_layers(lambda oc, ic, k: (oc, ic, k))
+    assert len(layers) == 52
+    hw, seen = {-1: 56}, Counter()
+    for i, ly in enumerate(layers):
+        src = i - 1 if ly.source is None else ly.source
+        assert -1 <= src < i
+        oc, ic, k = ly.weight
+        seen[(ic, hw[src], oc, k, ly.stride, ly.padding)] += 1
+        hw[i] = (hw[src] + 2 * ly.padding - k) // ly.stride + 1
+        if src >= 0:
+            assert layers[src].weight[0] == ic  # reads as many channels as its source writes
+    want = Counter({(s.C, s.H, s.K, s.KH, s.stride, s.pad): s.count for s in WL.RESNET50[1:]})
+    assert seen == want
