@@ -293,6 +293,27 @@ def main():
                                   pct_f16_peak=round(100 * gemm_ops / us_fp / 1e6 / PEAK_F16_TFLOPS, 2), kernel=v_fp,
                                   max_rel_err=float((np.abs(got - ref) / np.maximum(np.abs(ref), 1e-3 * np.abs(ref).max())).max()))
 
+    # the reference's own GEMM sizes (its drivers' constants): few output tiles, so the reduction is split between workgroups
+    ra = torch.randint(0, 256, (128, 768), dtype=torch.uint8, device=dev)
+    rw = torch.randint(-128, 128, (3072, 768), dtype=torch.int8, device=dev)
+    rc = torch.empty((128, 3072), dtype=torch.int32, device=dev)
+    us_r8 = time_us(lambda: _lib.check(L.unit_dense_u8s8s32(ra.data_ptr(), rw.data_ptr(), rc.data_ptr(), 128, 3072, 768, stream)),
+                    50, bursts=3)
+    v_r8 = U.last_variant()
+    rha = torch.randn((128, 3072), dtype=torch.float16, device=dev) / 55
+    rhb = torch.randn((3072, 768), dtype=torch.float16, device=dev)
+    rhc = torch.empty((128, 768), dtype=torch.float32, device=dev)
+    us_r16 = time_us(lambda: _lib.check(L.unit_gemm_f16(rha.data_ptr(), rhb.data_ptr(), rhc.data_ptr(), 128, 768, 3072, 0, stream)),
+                     50, bursts=3)
+    v_r16 = U.last_variant()
+    torch.cuda.synchronize()
+    want = rha.float() @ rhb.float()
+    gemm_ref_sizes = dict(
+        int8_dense_128x3072x768=dict(us=round(us_r8, 2), kernel=v_r8, source="apps/cpu/kernel/int8-gemm.py:9, apps/cpu/relay/int8-gemm.py:14-16"),
+        fp16_gemm_128x768x3072=dict(us=round(us_r16, 2), kernel=v_r16, source="apps/gpu/gemm.py:6",
+                                    max_rel_err=float(((rhc - want).abs() / want.abs().clamp_min(1e-3 * float(want.abs().max()))).max())))
+    del ra, rw, rc, rha, rhb, rhc, want
+
     # ------------------------------------------------------------------ secondary legs (BASELINE.json configs 0, 3, 4-fp16; layouts)
     def conv_i8_leg(shapes, batch, iters, fused=False, prepared=False, requant=False):
         rows, tot_us, tot_ops = [], 0.0, 0.0
@@ -590,6 +611,7 @@ def main():
         "cpu_baseline": cpu_baseline,
         "gemm_int8_4096": gemm_i8,
         "gemm_fp16_4096": gemm_f16,
+        "gemm_reference_sizes": gemm_ref_sizes,
         "mfma_probe": probe,
         "single_conv": single_conv,
         "resnet18_b1": resnet18_b1,

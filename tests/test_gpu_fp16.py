@@ -49,6 +49,23 @@ def test_gemm_fp16(dev, oracle, M, N, K, out_dtype):
     assert err <= (REL_TOL if out_dtype == "float32" else REL_TOL), (err, U.last_variant())
 
 
+@pytest.mark.parametrize("M,N,K", [(128, 768, 3072), (96, 200, 2056), (1, 8, 4096), (300, 260, 520)])
+def test_gemm_fp16_k_splits(dev, oracle, M, N, K):
+    """Few output tiles, long reduction (apps/gpu/gemm.py:6 is 128 x 768 x 3072): the reduction is shared between
+    workgroups that add into the zero-filled fp32 output; fp16 output keeps one workgroup per tile."""
+    a = rng.normal_f16((M, K), 131 + M, 1.0 / np.sqrt(K))
+    b = rng.normal_f16((K, N), 157 + N)
+    ta, tb = _t(a, dev), _t(b, dev)
+    ref = oracle.gemm_f16(a, b)
+    for operand in (tb, U.prepare_gemm_b(tb)):
+        out = U.gemm_fp16(ta, operand)
+        torch.cuda.synchronize()
+        assert int(U.last_variant().rsplit("_s", 1)[1]) > 1, U.last_variant()
+        assert max_rel(out.cpu().numpy(), ref) <= REL_TOL, U.last_variant()
+        half = U.gemm_fp16(ta, operand, "float16")
+        assert U.last_variant().endswith("_s1") and max_rel(half.cpu().numpy(), ref) <= REL_TOL
+
+
 PREPARED_GEMM_CASES = GEMM_CASES + [(4096, 4096, 1024), (2304, 2560, 192), (257, 260, 64), (3000, 2052, 200)]
 
 

@@ -68,6 +68,24 @@ def test_dense_packed_weights_direct_to_registers(dev, oracle, monkeypatch, M, N
     assert np.array_equal(out.cpu().numpy(), oracle.c_dense(a, wp)), U.last_variant()
 
 
+@pytest.mark.parametrize("M,N,K", [(128, 3072, 768), (50, 260, 1040), (1, 128, 8192)])
+def test_dense_k_splits_bit_exact(dev, oracle, M, N, K):
+    """Few output tiles: the reduction is shared between workgroups (int32 atomics, exact in any order); the output
+    buffer's previous contents must not leak into the sums."""
+    a = rng.uniform_u8((M, K), 500 + M)
+    w = rng.uniform_s8((N, K), 600 + N)
+    ref = oracle.dense_logical(a, w) if N % 128 else oracle.c_dense(a, oracle.prepack_dense_weight(w))
+    out = U.dense(_t(a, dev), _t(w, dev))
+    assert int(U.last_variant().rsplit("_s", 1)[1]) > 1, U.last_variant()
+    assert np.array_equal(out.cpu().numpy(), ref)
+    from unit_amd import _lib
+    garbage = torch.full((M, N), 12345, dtype=torch.int32, device=dev)
+    ta, tw = _t(a, dev), _t(w, dev)
+    _lib.check(_lib.load().unit_dense_u8s8s32(ta.data_ptr(), tw.data_ptr(), garbage.data_ptr(), M, N, K,
+                                              torch.cuda.current_stream().cuda_stream))
+    assert np.array_equal(garbage.cpu().numpy(), ref)
+
+
 def test_dense_largest_output(dev, oracle):
     """An output just below the 2^31-byte limit (23168^2 int32 = 2.147 GB): 32-bit offsets must not wrap."""
     M = N = 23168

@@ -76,7 +76,9 @@ struct DirectShape {
 // transposed through the wave's LDS scratch so that 64 lanes store 16 pixels x 64 bytes = 1 KiB of
 // consecutive output per instruction.  `wsb` (LDS, 32 values, or null) holds what is added per
 // channel before the scale: the 128 * sum(w) correction and / or the bias.
-template <class Op>
+// NCHW: planar (N, p.planar, OH, OW) output instead.  A template parameter and not a run-time branch:
+// the branch, unrolled into the four blocks of a one-wave tile, cost every layer 16 VGPRs and 4 % of its time.
+template <class Op, bool NCHW = false>
 __device__ __forceinline__ void store_block(const typename ConvEpilogue<Op>::Params &p, const typename Op::acc_t &acc,
                                             const int *wsb, int scale, int c0, int m0, int lane, char *scratch) {
   using out4_t = typename Op::out4_t;
@@ -84,7 +86,7 @@ __device__ __forceinline__ void store_block(const typename ConvEpilogue<Op>::Par
   constexpr int kPitch = 144;
   const int l32 = lane & 31, half = lane >> 5;
   const int rp = lane >> 2, piece = lane & 3;
-  if (p.planar) {
+  if constexpr (NCHW) {
     // (N, planar, OH, OW): register r of a lane is channel 8 (r / 4) + 4 half + r % 4 of the lane's pixel, so
     // a register of 32 lanes is 128 consecutive bytes of one channel plane: no transpose
     const int m = m0 + l32;
@@ -195,7 +197,7 @@ __device__ __forceinline__ void store_block_q8(const typename ConvEpilogue<Op>::
   }
 }
 
-template <class Op, class S, bool SHIFT, bool PREP = false, bool C4 = false, bool Q8 = false>
+template <class Op, class S, bool SHIFT, bool PREP = false, bool C4 = false, bool Q8 = false, bool NCHW = false>
 __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ data, const char *__restrict__ wgt,
                                                      typename ConvEpilogue<Op>::Params ep, ConvGeom g, GridMap gm) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -206,6 +208,7 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
   static_assert(kInt || (!SHIFT && !S::PAD), "the fp16 operator has neither a shift nor padding");
   static_assert(!C4 || (kInt && S::PAD), "4-channel blocks: int8, masked loads");
   static_assert(!Q8 || kInt, "requantised output is an int8 operator");
+  static_assert(!NCHW || (kInt && !Q8), "planar output: the int32 fused form");
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int l32 = lane & 31, half = lane >> 5;
@@ -501,7 +504,7 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
         if constexpr (Q8)
           store_block_q8<Op>(ep, acc[i][j], addend ? wsum + i * 32 : nullptr, x0 + i * 32, y0 + j * 32, lane);
         else
-          store_block<Op>(ep, acc[i][j], addend ? wsum + i * 32 : nullptr, ep.scale, x0 + i * 32, y0 + j * 32, lane,
+          store_block<Op, NCHW>(ep, acc[i][j], addend ? wsum + i * 32 : nullptr, ep.scale, x0 + i * 32, y0 + j * 32, lane,
                           scratch);
   } else if constexpr (!kParked) {
     // sum the partial tiles of the KG waves in LDS, then share the blocks among the waves
@@ -528,7 +531,7 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
       if constexpr (Q8)
         store_block_q8<Op>(ep, total, addend ? wsum + i * 32 : nullptr, x0 + i * 32, y0 + j * 32, lane);
       else
-        store_block<Op>(ep, total, addend ? wsum + i * 32 : nullptr, ep.scale, x0 + i * 32, y0 + j * 32, lane, scratch);
+        store_block<Op, NCHW>(ep, total, addend ? wsum + i * 32 : nullptr, ep.scale, x0 + i * 32, y0 + j * 32, lane, scratch);
     }
   } else {
     // every wave parks its partial tile (and addends); the owner of a block adds them in wave order
@@ -570,10 +573,10 @@ __global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ da
           for (int w = 0; w < KG; ++w) a += wsum[w * (TX * 32) + i * 32 + l32];
           reinterpret_cast<int *>(scratch)[1152 + l32] = a;  // behind the transpose area
         }
-        store_block<Op>(ep, total, addend ? reinterpret_cast<const int *>(scratch) + 1152 : nullptr, ep.scale,
+        store_block<Op, NCHW>(ep, total, addend ? reinterpret_cast<const int *>(scratch) + 1152 : nullptr, ep.scale,
                         x0 + i * 32, y0 + j * 32, lane, scratch);
       } else {
-        store_block<Op>(ep, total, nullptr, 1, x0 + i * 32, y0 + j * 32, lane, scratch);
+        store_block<Op, NCHW>(ep, total, nullptr, 1, x0 + i * 32, y0 + j * 32, lane, scratch);
       }
     }
   }

@@ -5,14 +5,14 @@
 
 namespace unit {
 
-template <class Op, class S, bool SHIFT, bool PREP = false, bool C4 = false, bool Q8 = false>
+template <class Op, class S, bool SHIFT, bool PREP = false, bool C4 = false, bool Q8 = false, bool NCHW = false>
 int run_direct(const char *what, const char *tag, const unit_conv_desc *d, const ConvGeom &g, const void *data,
                const void *w, const int *bias, int scale, void *out, const ConvPlan &plan, hipStream_t s,
                const int *bias2 = nullptr, int shift = 0, int planar = 0) {
   const int ntab = C4 ? 2 * g.c4_steps : (Op::kInt ? 2 * ((g.ntaps + 1) / 2) : g.ntaps);
   const int lds = S::template lds_fixed<Op>() + ntab * 8;
   if (lds > kMaxLds) return fail(UNIT_E_ARG, "%s: needs %d bytes of LDS (limit %d)", what, lds, kMaxLds);
-  auto kern = conv_direct<Op, S, SHIFT, PREP, C4, Q8>;
+  auto kern = conv_direct<Op, S, SHIFT, PREP, C4, Q8, NCHW>;
   static thread_local int lds_allowed = 0;  // the opt-in for > 64 KiB of dynamic LDS is sticky per kernel
   if (lds > lds_allowed) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),

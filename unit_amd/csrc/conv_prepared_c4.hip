@@ -13,10 +13,14 @@ int conv_c4_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGe
 #define UNIT_CONV_VARIANT(ID, BX, BY, BKB, WX, WY, PF, FF, KG)
 #define UNIT_CONV_DIRECT(ID, TX, TY, KG, D)                                                                            \
   case ID:                                                                                                             \
-    return shift ? run_direct<OpI8, DirectShape<TX, TY, KG, D, true>, true, true, true>(what, "i8prep_c4", d, g, data, \
-                                                                                         w, addend, 1, out, plan, s)   \
-                 : run_direct<OpI8, DirectShape<TX, TY, KG, D, true>, false, true, true>(                              \
-                       what, tag, d, g, data, w, addend, scale, out, plan, s, nullptr, 0, planar);
+    if (shift)                                                                                                         \
+      return run_direct<OpI8, DirectShape<TX, TY, KG, D, true>, true, true, true>(what, "i8prep_c4", d, g, data, w,    \
+                                                                                  addend, 1, out, plan, s);            \
+    if (planar)                                                                                                        \
+      return run_direct<OpI8, DirectShape<TX, TY, KG, D, true>, false, true, true, false, true>(                       \
+          what, tag, d, g, data, w, addend, scale, out, plan, s, nullptr, 0, planar);                                  \
+    return run_direct<OpI8, DirectShape<TX, TY, KG, D, true>, false, true, true>(what, tag, d, g, data, w, addend,     \
+                                                                                 scale, out, plan, s);
   switch (plan.variant) {
 #include "conv_variants.def"
     default:

@@ -68,8 +68,10 @@ int run_gemm_f16_bt(const void *a, const void *bt, void *c, int M, int N, int K,
   typename YL::Params yp{static_cast<const char *>(bt), N, K * 2, K * 2};
   typename Epi::Params ep{c, M, N};
   const int nk = ceil_div(K * 2, T::BKB), gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
-  set_variant("f16gemmbt_x%d_y%d_k%d_w%dx%d%s", T::BX, T::BY, T::BKB, T::WX, T::WY, OUT_F16 ? "_h" : "");
-  return launch_mma<OpF16, T, XL, YL, Epi, WS_NONE>(xp, yp, ep, nk, gx, gy, 4, 1, c, 0, 0, s, "unit_gemm_f16_prepared");
+  const int splits = OUT_F16 ? 1 : gemm_k_splits("UNIT_AMD_GEMM_F16_SPLITK", gx * gy, nk);
+  set_variant("f16gemmbt_x%d_y%d_k%d_w%dx%d%s_s%d", T::BX, T::BY, T::BKB, T::WX, T::WY, OUT_F16 ? "_h" : "", splits);
+  return launch_mma<OpF16, T, XL, YL, Epi, WS_NONE>(xp, yp, ep, nk, gx, gy, 4, splits, c, (size_t)M * N * 4, 0, s,
+                                                    "unit_gemm_f16_prepared");
 }
 
 template <bool OUT_F16>
@@ -105,9 +107,11 @@ int run_gemm_f16(const void *a, const void *b, void *c, int M, int N, int K, hip
   typename YL::Params yp{static_cast<const char *>(b), N, K, N + 4, 0, N * 2};
   typename Epi::Params ep{c, M, N};
   const int nk = ceil_div(K * 2, T::BKB), gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
-  set_variant("f16gemm_x%d_y%d_k%d_w%dx%d_p%d%s%s", T::BX, T::BY, T::BKB, T::WX, T::WY, PF, TAIL ? "" : "e",
-              OUT_F16 ? "_h" : "");
-  return launch_mma<OpF16, T, XL, YL, Epi, WS_NONE>(xp, yp, ep, nk, gx, gy, 4, 1, c, 0, 0, s, "unit_gemm_f16");
+  const int splits = OUT_F16 ? 1 : gemm_k_splits("UNIT_AMD_GEMM_F16_SPLITK", gx * gy, nk);
+  set_variant("f16gemm_x%d_y%d_k%d_w%dx%d_p%d%s%s_s%d", T::BX, T::BY, T::BKB, T::WX, T::WY, PF, TAIL ? "" : "e",
+              OUT_F16 ? "_h" : "", splits);
+  return launch_mma<OpF16, T, XL, YL, Epi, WS_NONE>(xp, yp, ep, nk, gx, gy, 4, splits, c, (size_t)M * N * 4, 0, s,
+                                                    "unit_gemm_f16");
 }
 
 template <bool OUT_F16>

@@ -54,6 +54,21 @@ inline int check_aligned(const char *what, std::initializer_list<const void *> p
   return UNIT_OK;
 }
 
+// k-splits of a GEMM.  Few output tiles and a long reduction leave most of the chip idle (the reference's own
+// GEMM sizes, 128 x 768 x 3072 in apps/gpu/gemm.py:6 and 128 x 3072 x 768 in apps/cpu/kernel/int8-gemm.py:9, are 6
+// and 24 tiles of 128 x 128; the reference splits the reduction of the first with rfactor, gemm.py:22-40): the
+// reduction is then shared between workgroups that add their partial tiles with atomics into the zero-filled
+// output, about 128 workgroups in all and at least four stages each.  Exact for int32; for fp32 the order of the
+// additions varies from run to run (last-bit differences).  The environment variable pins the count (1 = off).
+inline int gemm_k_splits(const char *env, int tiles, int nk) {
+  int splits = tuning_override(env);
+  if (splits <= 0) {
+    splits = 1;
+    if (tiles < 128) splits = 128 / tiles < nk / 4 ? 128 / tiles : nk / 4;
+  }
+  return splits < 1 ? 1 : (splits > nk ? nk : splits);
+}
+
 // Enqueue mma_kernel over gx x gy tiles and `splits` k-ranges.  With splits > 1 the epilogue
 // accumulates with atomics, so `out` (out_bytes, a multiple of 16) is zero-filled first.
 template <class Op, class T, class XL, class YL, class Epi, int WS>
