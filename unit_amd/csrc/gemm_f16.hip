@@ -68,7 +68,7 @@ int run_gemm_f16_bt(const void *a, const void *bt, void *c, int M, int N, int K,
   typename YL::Params yp{static_cast<const char *>(bt), N, K * 2, K * 2};
   typename Epi::Params ep{c, M, N};
   const int nk = ceil_div(K * 2, T::BKB), gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
-  const int splits = OUT_F16 ? 1 : gemm_k_splits("UNIT_AMD_GEMM_F16_SPLITK", gx * gy, nk);
+  const int splits = OUT_F16 ? 1 : gemm_k_splits("UNIT_AMD_GEMM_F16_SPLITK", M, N, 2l * K, nk);
   set_variant("f16gemmbt_x%d_y%d_k%d_w%dx%d%s_s%d", T::BX, T::BY, T::BKB, T::WX, T::WY, OUT_F16 ? "_h" : "", splits);
   return launch_mma<OpF16, T, XL, YL, Epi, WS_NONE>(xp, yp, ep, nk, gx, gy, 4, splits, c, (size_t)M * N * 4, 0, s,
                                                     "unit_gemm_f16_prepared");
@@ -107,7 +107,7 @@ int run_gemm_f16(const void *a, const void *b, void *c, int M, int N, int K, hip
   typename YL::Params yp{static_cast<const char *>(b), N, K, N + 4, 0, N * 2};
   typename Epi::Params ep{c, M, N};
   const int nk = ceil_div(K * 2, T::BKB), gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
-  const int splits = OUT_F16 ? 1 : gemm_k_splits("UNIT_AMD_GEMM_F16_SPLITK", gx * gy, nk);
+  const int splits = OUT_F16 ? 1 : gemm_k_splits("UNIT_AMD_GEMM_F16_SPLITK", M, N, 2l * K, nk);
   set_variant("f16gemm_x%d_y%d_k%d_w%dx%d_p%d%s%s_s%d", T::BX, T::BY, T::BKB, T::WX, T::WY, PF, TAIL ? "" : "e",
               OUT_F16 ? "_h" : "", splits);
   return launch_mma<OpF16, T, XL, YL, Epi, WS_NONE>(xp, yp, ep, nk, gx, gy, 4, splits, c, (size_t)M * N * 4, 0, s,
@@ -137,6 +137,8 @@ int gemm_f16(const void *a, const void *b, void *c, int M, int N, int K, hipStre
     // 64 (m) x 128 (n) wave tiles: measured 8-10 % faster than 128 x 64 (512-byte row runs per wave in the write-back)
     return run_gemm_f16<Tile<256, 256, 128, 4, 2>, OUT_F16>(a, b, c, M, N, K, s);
   }
+  // mid sizes: 128 x 256 tiles of eight waves (measured 8-12 % faster than 128 x 128 at 2048^3, 1024 x 4096 x 4096)
+  if (M >= 128 && N >= 256 && K >= 128) return run_gemm_f16<Tile<128, 256, 128, 4, 2>, OUT_F16>(a, b, c, M, N, K, s);
   return run_gemm_f16<Tile<128, 128, 64, 2, 2>, OUT_F16>(a, b, c, M, N, K, s);
 }
 

@@ -20,7 +20,7 @@ int run_dense(const void *a, const void *w, void *c, int M, int N, int K, hipStr
   typename Epi::Params ep{c, M, N};
   const int nk = ceil_div(K, T::BKB), gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
   // few tiles and a long reduction: share K between workgroups (int32 atomics are exact)
-  int splits = gemm_k_splits("UNIT_AMD_DENSE_SPLITK", gx * gy, nk);
+  int splits = gemm_k_splits("UNIT_AMD_DENSE_SPLITK", M, N, K, nk);
   if ((size_t)M * N * 4 % 16) splits = 1;
   set_variant("i8dense%s_x%d_y%d_k%d_w%d%s_s%d", PACKED ? "pk" : "rm", T::BX, T::BY, T::BKB, T::NT / 64, TAIL ? "" : "e",
               splits);

@@ -58,13 +58,20 @@ inline int check_aligned(const char *what, std::initializer_list<const void *> p
 // GEMM sizes, 128 x 768 x 3072 in apps/gpu/gemm.py:6 and 128 x 3072 x 768 in apps/cpu/kernel/int8-gemm.py:9, are 6
 // and 24 tiles of 128 x 128; the reference splits the reduction of the first with rfactor, gemm.py:22-40): the
 // reduction is then shared between workgroups that add their partial tiles with atomics into the zero-filled
-// output, about 128 workgroups in all and at least four stages each.  Exact for int32; for fp32 the order of the
-// additions varies from run to run (last-bit differences).  The environment variable pins the count (1 = off).
-inline int gemm_k_splits(const char *env, int tiles, int nk) {
+// output.  Below 128 tiles of 128 x 128: about 128 workgroups in all, at least 256 reduction bytes each; up to
+// 256 tiles, three splits when each still gets 2 KiB of reduction (measured: 256 x 8192 x 8192 fp16 133 -> 67 us).
+// More tiles fill the chip by themselves, and the atomics (output bytes x splits) then cost more than they gain.
+// Exact for int32; for fp32 the order of the additions varies from run to run (last-bit differences).
+// The environment variable pins the count (1 = off).  kbytes: reduction bytes per row; nk: stages of the tile.
+inline int gemm_k_splits(const char *env, int M, int N, long kbytes, int nk) {
   int splits = tuning_override(env);
   if (splits <= 0) {
+    const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
     splits = 1;
-    if (tiles < 128) splits = 128 / tiles < nk / 4 ? 128 / tiles : nk / 4;
+    if (tiles < 128)
+      splits = (int)(128 / tiles < kbytes / 256 ? 128 / tiles : kbytes / 256);
+    else if (tiles < 256 && kbytes >= 6144)
+      splits = 3;
   }
   return splits < 1 ? 1 : (splits > nk ? nk : splits);
 }
