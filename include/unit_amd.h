@@ -120,7 +120,7 @@ int unit_dense_dotprod_u8s8s32(const void *a, const void *wp, void *c, int32_t M
 
 /* relay.nn.dense(x, w, out_dtype='int32') of apps/cpu/relay/int8-gemm.py:14-16 on the
  * un-packed weight:  a u8 (M, K), w s8 (N, K) row-major, c i32 (M, N) = a . w^T.
- * K % 16 == 0. */
+ * K % 16 == 0.  Few output tiles: the reduction is split between workgroups (int32 atomics, exact). */
 int unit_dense_u8s8s32(const void *a, const void *w, void *c, int32_t M, int32_t N, int32_t K,
                        unit_stream_t stream);
 
@@ -130,7 +130,11 @@ int unit_dense_u8s8s32(const void *a, const void *w, void *c, int32_t M, int32_t
  *   c[x][y] = sum_k f32(a[x][k]) * f32(b[k][y]),  a f16 (M, K), b f16 (K, N), row-major;
  * c is f32 when out_f16 == 0, else f16 (round-to-nearest-even of the fp32 sum).
  * K % 8 == 0, N % 4 == 0.  Replaces wmma.m16n16k16 (python/tensorizer/intrinsics/gpu.py:104-216)
- * with v_mfma_f32_32x32x16_f16. */
+ * with v_mfma_f32_32x32x16_f16.  With few output tiles and a long reduction (the script's own
+ * 128 x 768 x 3072) and f32 output, the reduction is split between workgroups as the reference's
+ * rfactor schedule does (apps/gpu/gemm.py:22-40): partial tiles are added into the zero-filled c,
+ * so the summation order, and with it the last bits of c, can differ from run to run
+ * (UNIT_AMD_GEMM_F16_SPLITK=1 keeps one workgroup per tile). */
 int unit_gemm_f16(const void *a, const void *b, void *c, int32_t M, int32_t N, int32_t K,
                   int32_t out_f16, unit_stream_t stream);
 
