@@ -47,12 +47,20 @@ namespace unit {
 
 // PAD: the convolution has zero padding, so taps can fall outside the image and are masked per
 // lane; without it every tap of every valid pixel lies inside and the masking code is left out.
+// D_ = ring depth, + 16 when the kernel is to be built for four waves per SIMD.
 template <int TX_, int TY_, int KG_, int D_, bool PAD_ = true>
 struct DirectShape {
-  static constexpr int TX = TX_, TY = TY_, KG = KG_, D = D_;
+  static constexpr int TX = TX_, TY = TY_, KG = KG_, D = D_ % 16;
   static constexpr bool PAD = PAD_;
   static constexpr int BX = TX * 32, BY = TY * 32;
   static constexpr int NT = 64 * KG;
+  // One wave per tile and a two-deep ring: asked for four waves per SIMD the register allocator fits the kernel
+  // into 128 VGPRs without spilling (it settles at 140 = three waves otherwise).  Deeper rings, wider tiles and
+  // the per-tap loads of the reference's weight layout or of 4-channel blocks spill; the kernel asks only with
+  // PREP && !C4.  A variant of its own, because it is not always a gain: short reductions with small outputs
+  // run 0.6-0.9 us faster, the output-bound 1 x 1 64 -> 256 @56 layer 2 us slower.
+  static constexpr bool kFourWaves = D_ >= 16;  // the variant asks for it (shown as "w4" in the variant name)
+  static constexpr int kMinWavesPerSimd = (D_ >= 16 && KG == 1 && D == 2 && TX == 2 && TY == 2) ? 4 : 1;
   static constexpr int kScratch = 32 * 144 + 128;  // per wave: transpose area (32 pixels x 144-byte pitch) + 32 addends
   static constexpr int TILE = TX * TY * 4096;     // one 4-byte accumulator tile
   static constexpr int WSUM = TX * 32 * 4;        // summed 128 * weight sums
@@ -198,7 +206,7 @@ __device__ __forceinline__ void store_block_q8(const typename ConvEpilogue<Op>::
 }
 
 template <class Op, class S, bool SHIFT, bool PREP = false, bool C4 = false, bool Q8 = false, bool NCHW = false>
-__global__ __launch_bounds__(S::NT) void conv_direct(const char *__restrict__ data, const char *__restrict__ wgt,
+__global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !C4 ? S::kMinWavesPerSimd : 1))) void conv_direct(const char *__restrict__ data, const char *__restrict__ wgt,
                                                      typename ConvEpilogue<Op>::Params ep, ConvGeom g, GridMap gm) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   constexpr int TX = S::TX, TY = S::TY, KG = S::KG, D = S::D;

@@ -30,7 +30,8 @@ int run_direct(const char *what, const char *tag, const unit_conv_desc *d, const
   gm.total = gm.gx * gm.gy;
   char tail[16] = "";
   if (panel) snprintf(tail, sizeof tail, "_r%d", panel);
-  set_variant("%s_x%d_y%d_g%d_d%d%s%s_s1", tag, S::BX, S::BY, S::KG, S::D, S::PAD ? "" : "n", tail);
+  set_variant("%s_x%d_y%d_g%d_d%d%s%s%s_s1", tag, S::BX, S::BY, S::KG, S::D,
+              S::kFourWaves ? "w4" : "", S::PAD ? "" : "n", tail);
   hipLaunchKernelGGL(kern, dim3(gm.total), dim3(S::NT), lds, s, static_cast<const char *>(data),
                      static_cast<const char *>(w), ep, g, gm);
   hipError_t e = hipGetLastError();

@@ -18,7 +18,7 @@ struct TileShape {
 // index = variant id used by the tuning table and UNIT_AMD_CONV_VARIANT (1-based there)
 constexpr TileShape kConvTiles[] = {
 #define UNIT_CONV_VARIANT(ID, BX, BY, BKB, WX, WY, PF, FF, KG) {BX, BY, BKB, (WX) * (WY) * (KG), PF, FF, KG, false},
-#define UNIT_CONV_DIRECT(ID, TX, TY, KG, D) {(TX) * 32, (TY) * 32, 32, KG, D, false, KG, true},
+#define UNIT_CONV_DIRECT(ID, TX, TY, KG, D) {(TX) * 32, (TY) * 32, 32, KG, (D) % 16, false, KG, true},
 #include "conv_variants.def"
 #undef UNIT_CONV_DIRECT
 #undef UNIT_CONV_VARIANT
