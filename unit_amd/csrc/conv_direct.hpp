@@ -210,6 +210,13 @@ __global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !
                                                      typename ConvEpilogue<Op>::Params ep, ConvGeom g, GridMap gm) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   constexpr int TX = S::TX, TY = S::TY, KG = S::KG, D = S::D;
+  {
+    // Touch every 64-byte line of the 260 bytes of kernel arguments at once: the compiler fetches the arguments
+    // where it first needs them, in three dependent rounds of scalar loads before the first operand fetch.
+    const auto *ka = (const __attribute__((address_space(4))) int *)__builtin_amdgcn_kernarg_segment_ptr();
+    const int w0 = ka[0], w1 = ka[16], w2 = ka[32], w3 = ka[48], w4 = ka[64];
+    asm volatile("" ::"s"(w0), "s"(w1), "s"(w2), "s"(w3), "s"(w4));
+  }
   constexpr bool kInt = Op::kInt;
   constexpr int TAPB = C4 ? 4 : (kInt ? 16 : 32);  // bytes of one pixel and tap
   constexpr int WTAP = kInt ? 256 : 512;           // bytes of one tap of a 16-channel weight block
