@@ -569,15 +569,37 @@ def main():
         g_rm()
         torch.cuda.synchronize()
         rows = 512
-        ref = O.c_dense(a8[:rows].cpu().numpy(), O.prepack_dense_weight(w8_np), nthreads=cores)
+        a8_rows, wp8_np = a8[:rows].cpu().numpy(), O.prepack_dense_weight(w8_np)
+        ref = O.c_dense(a8_rows, wp8_np, nthreads=cores)
         if not np.array_equal(c8[:rows].cpu().numpy(), ref):
             bit_exact = False
             print("bench.py: MISMATCH vs oracle in int8 GEMM", file=sys.stderr)
+        # the GEMM configs on the host, on a bounded sample (512 of the 4096 rows of a, all of b), the reference's
+        # number=10 protocol (apps/cpu/kernel/int8-gemm.py:34): int8 by the VNNI oracle, fp16 as an fp32 GEMM of the
+        # fp16-rounded operands (torch CPU matmul); and the host's vpdpbusd peak, as poc/vnni/micro.cc measures it
+        t1 = time.perf_counter()
+        for _ in range(10):
+            O.c_dense(a8_rows, wp8_np, nthreads=cores)
+        cpu_i8_s = (time.perf_counter() - t1) / 10
+        af32, bf32 = torch.from_numpy(ah_np[:rows].astype(np.float32)), torch.from_numpy(bh_np.astype(np.float32))
+        torch.matmul(af32, bf32)
+        t1 = time.perf_counter()
+        for _ in range(10):
+            torch.matmul(af32, bf32)
+        cpu_f16_s = (time.perf_counter() - t1) / 10
+        vnni_peak = O.vnni_peak_gops(nthreads=cores) / 1e3 if O.has_vnni() else None
         cpu_baseline = dict(value=round(step_ops / cpu_s / 1e12, 4), unit="TOP/s", cores=cores, kind="port",
                             vnni=bool(O.has_vnni()),
                             sample="the same step (53 convolutions, batch 32) by the AVX-512 VNNI oracle: each of "
                                    "the 20 unique layers repeated for about 0.5 s, mean time x its multiplicity",
-                            seconds=round(cpu_s, 3))
+                            seconds=round(cpu_s, 3),
+                            host_vnni_peak_tops=None if vnni_peak is None else round(vnni_peak, 3),
+                            pct_of_host_vnni_peak=None if not vnni_peak else round(100 * step_ops / cpu_s / 1e12 / vnni_peak, 1),
+                            gemm_int8_4096=dict(tops=round(2.0 * rows * N * K / cpu_i8_s / 1e12, 3),
+                                                sample=f"{rows} of the 4096 rows of a, mean of 10 runs, VNNI oracle"),
+                            gemm_fp16_4096=dict(tflops=round(2.0 * rows * N * K / cpu_f16_s / 1e12, 3),
+                                                sample=f"{rows} of the 4096 rows of a, mean of 10 runs, torch CPU fp32 matmul "
+                                                       "of the fp16-rounded operands"))
         gemm_i8["bit_exact_rows_checked"] = rows
 
     line = {
