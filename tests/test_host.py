@@ -95,3 +95,28 @@ def test_resnet50_chain_lists_the_logged_shapes():
             assert layers[src].weight[0] == ic  # reads as many channels as its source writes
     want = Counter({(s.C, s.H, s.K, s.KH, s.stride, s.pad): s.count for s in WL.RESNET50[1:]})
     assert seen == want
+
+
+def test_tuned_tables_name_existing_variants():
+    """Every row of the tuned tables compiled into the library names a kernel variant that exists; the tables for
+    prepared weights only name direct variants (the only ones that read the prepared layout)."""
+    import glob
+    import os
+    import re
+    from unit_amd import _lib
+    L = _lib.load()
+    count = L.unit_conv_variant_count()
+    csrc = os.path.join(os.path.dirname(os.path.abspath(U.__file__)), "csrc")
+    files = sorted(glob.glob(os.path.join(csrc, "tuned_conv_*.inc")))
+    assert len(files) == 4
+    for path in files:
+        rows = re.findall(r"\{([^}]*)\}", open(path).read())
+        assert rows, path
+        keys = set()
+        for row in rows:
+            npix, k, c, kh, kw, sh, variant, splits, panel = (int(v) for v in row.split(","))
+            assert 0 <= variant < count and splits >= 1 and panel >= 0, (path, row)
+            assert (npix, k, c, kh, kw, sh) not in keys, (path, row)  # one choice per shape
+            keys.add((npix, k, c, kh, kw, sh))
+            if path.endswith("_prepared.inc"):
+                assert L.unit_conv_variant_is_direct(variant) == 1, (path, row)
