@@ -474,22 +474,15 @@ __global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !
       __builtin_amdgcn_sched_barrier(0);
     });
     int s = s0;
-    for (; s + 2 * D <= s1; s += D)
+    // while more than D k-steps remain: consume a round and fetch the next one (in the last round fewer than D
+    // k-steps are new; the surplus fetches repeat the wave's last k-step)
+    for (; s + D < s1; s += D)
       for_slots([&](auto u) __attribute__((always_inline)) {
         consume(u);
         __builtin_amdgcn_sched_barrier(0);
         fetch(u);
         __builtin_amdgcn_sched_barrier(0);
       });
-    if (s + D < s1) {  // D < remaining < 2 D: one more round of fetches (the surplus ones repeat the last k-step)
-      for_slots([&](auto u) __attribute__((always_inline)) {
-        consume(u);
-        __builtin_amdgcn_sched_barrier(0);
-        fetch(u);
-        __builtin_amdgcn_sched_barrier(0);
-      });
-      s += D;
-    }
     for_slots([&](auto u) __attribute__((always_inline)) {  // 1 .. D k-steps left, all in flight
       if (s + decltype(u)::value < s1) consume(u);
       __builtin_amdgcn_sched_barrier(0);
