@@ -130,4 +130,17 @@ def test_planar_needs_prepared_weights_and_a_matching_channel_count(dev):
 
 def test_driver_prints_a_time(dev, capsys):
     assert relay.main("1 32 14 14 32 32 3 3 1 1".split()) == 0
-    assert " us " in capsys.readouterr().out
+    out = capsys.readouterr().out
+    assert " us per run" in out
+
+
+def test_graph_replay_follows_the_input(dev):
+    wt = rng.uniform_s8((32, 16, 3, 3), 31)
+    g = relay.Conv2dBiasMultiply(torch.from_numpy(wt).to(dev), None, 5, 1, 1)
+    x1, x2 = rng.uniform_s8((2, 16, 9, 9), 32), rng.uniform_s8((2, 16, 9, 9), 33)
+    xd = torch.from_numpy(x1).to(dev)
+    replay = g.graph(xd)
+    for x in (x1, x2, x1):  # eager work and synchronisations between the replays
+        xd.copy_(torch.from_numpy(x).to(dev))
+        torch.cuda.synchronize()
+        assert np.array_equal(replay().cpu().numpy(), _plain_graph(x, wt, None, 5, 1, 1))
