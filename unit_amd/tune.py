@@ -10,7 +10,7 @@ library's planner consults first (rebuild after tuning).  Needs an MI355X.  With
 convolutions on prepared weights are tuned (direct variants only) into
 tuned_conv_{i8,f16}_prepared.inc.
 
-    python -m unit_amd.tune [--dtype i8|f16] [--prepared] [--nets resnet50:32,resnet18:1] [--iters 20] [--write]
+    python -m unit_amd.tune [--dtype i8|f16] [--prepared] [--nets resnet50:32,resnet18:1] [--iters 20] [--instances 8] [--write]
 """
 import argparse
 import ctypes
@@ -30,7 +30,7 @@ def _shapes(spec):
     return out
 
 
-def tune(spec, iters=20, verbose=True, dtype="i8", prepared=False):
+def tune(spec, iters=20, verbose=True, dtype="i8", prepared=False, instances=1):
     import torch
 
     from . import _lib, last_variant
@@ -94,12 +94,26 @@ def tune(spec, iters=20, verbose=True, dtype="i8", prepared=False):
                 wt = prepare_conv2d_weight(wt).buf
                 entry = L.unit_conv2d_nchwc_u8s8s32_prepared if dtype == "i8" else L.unit_conv2d_nchw16c_f16f32_prepared
 
+            # instances > 1: the launches cycle through that many copies of the layer's tensors, so that a launch
+            # finds its operands the way a layer of a running network does (last touched many launches ago), not
+            # in the caches its own previous launch filled
+            if instances < 0:  # as many copies as fill -instances MiB (at most 64): more than the memory-side cache holds
+                per = data.numel() * data.element_size() + wt.numel() * wt.element_size() + out.numel() * out.element_size()
+                n_inst = max(1, min(64, -(instances * (1 << 20)) // per + 1))
+            else:
+                n_inst = instances
+            copies = [(data, wt, out)] + [(data.clone(), wt.clone(), torch.empty_like(out)) for _ in range(n_inst - 1)]
+            turn = [0]
+
             def call():
-                return entry(ctypes.byref(desc), data.data_ptr(), wt.data_ptr(), out.data_ptr(), stream)
+                d_, w_, o_ = copies[turn[0] % n_inst]
+                turn[0] += 1
+                return entry(ctypes.byref(desc), d_.data_ptr(), w_.data_ptr(), o_.data_ptr(), stream)
 
             os.environ["UNIT_AMD_CONV_VARIANT"] = "0"
             os.environ["UNIT_AMD_CONV_SPLITK"] = "0"
             os.environ["UNIT_AMD_CONV_PANEL"] = "0"
+            turn[0] = 0
             _lib.check(call())
             torch.cuda.synchronize()
             ref = out.clone()
@@ -119,6 +133,7 @@ def tune(spec, iters=20, verbose=True, dtype="i8", prepared=False):
                     os.environ["UNIT_AMD_CONV_SPLITK"] = str(splits)
                     os.environ["UNIT_AMD_CONV_PANEL"] = str(panel)
                     out.fill_(-7)
+                    turn[0] = 0  # the checked launch writes `out`
                     if call() != 0:  # variant cannot run this shape (LDS budget)
                         break
                     torch.cuda.synchronize()
@@ -167,11 +182,14 @@ def main():
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--dtype", default="i8", choices=["i8", "f16"])
     ap.add_argument("--prepared", action="store_true", help="tune the convolutions on prepared weights")
+    ap.add_argument("--instances", type=int, default=1,
+                    help="cycle the timed launches through this many copies of each layer's tensors (cold operands); "
+                         "-M: as many copies as fill M MiB, at most 64")
     ap.add_argument("--write", action="store_true", help="rewrite csrc/tuned_conv_<dtype>[_prepared].inc")
     ap.add_argument("--table", default=None, help="write the table here instead of csrc/tuned_conv_i8.inc")
     ap.add_argument("--json", default=None, help="also dump the raw results here")
     args = ap.parse_args()
-    results = tune(args.nets, args.iters, dtype=args.dtype, prepared=args.prepared)
+    results = tune(args.nets, args.iters, dtype=args.dtype, prepared=args.prepared, instances=args.instances)
     if args.json:
         json.dump(results, open(args.json, "w"), indent=1)
     if args.write or args.table:
