@@ -60,7 +60,8 @@ struct DirectShape {
   // PREP && !C4.  A variant of its own, because it is not always a gain: short reductions with small outputs
   // run 0.6-0.9 us faster, the output-bound 1 x 1 64 -> 256 @56 layer 2 us slower.
   static constexpr bool kFourWaves = D_ >= 16;  // the variant asks for it (shown as "w4" in the variant name)
-  static constexpr int kMinWavesPerSimd = (D_ >= 16 && KG == 1 && D == 2 && TX == 2 && TY == 2) ? 4 : 1;
+  static constexpr int kMinWavesPerSimd =
+      (D_ >= 16 && KG == 1 && TX == 2 && TY == 2 && (D == 2 || (D == 3 && !PAD))) ? 4 : 1;  // three-deep: 127 VGPRs unpadded
   static constexpr int kScratch = 32 * 144 + 128;  // per wave: transpose area (32 pixels x 144-byte pitch) + 32 addends
   static constexpr int TILE = TX * TY * 4096;     // one 4-byte accumulator tile
   static constexpr int WSUM = TX * 32 * 4;        // summed 128 * weight sums
