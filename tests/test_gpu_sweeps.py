@@ -1,0 +1,49 @@
+"""The benchmark sweeps at their full sizes, every layer bit-exact against the VNNI oracle: ResNet-18 at batch 1 and
+ResNet-50 at batch 32 (BASELINE configs 3 and 4; shapes of cpu-shapes.log:368-420), on the reference's weight layout and
+on prepared weights."""
+import numpy as np
+import pytest
+import torch
+
+import unit_amd as U
+from unit_amd import rng
+from unit_amd import workloads as WL
+
+pytestmark = pytest.mark.gpu
+
+
+def _t(a, dev):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def _layer(s, batch, seed):
+    cb = WL.channel_block(s.C)
+    cp = -(-s.C // cb) * cb
+    data = rng.uniform_u8((batch, cp // cb, s.H, s.W, cb), seed)
+    if cp != s.C:
+        data[..., s.C % cb:] = 0  # padded input channels hold zeros
+    wt = rng.uniform_s8((s.K // 16, cp // cb, s.KH, s.KW, cb // 4, 16, 4), seed + 1)
+    return data, wt
+
+
+@pytest.mark.parametrize("s", WL.RESNET18, ids=lambda s: s.name)
+def test_resnet18_batch1_layer(dev, oracle, s):
+    data, wt = _layer(s, 1, 7000 + s.C + s.K)
+    ref = oracle.c_conv2d_nchwc(data, wt, s.stride, s.pad, 1)
+    td, tw = _t(data, dev), _t(wt, dev)
+    assert np.array_equal(U.conv2d_NCHWc_int8(td, tw, s.stride, s.pad).cpu().numpy(), ref), U.last_variant()
+    if WL.channel_block(s.C) == 16 or s.KW <= 8:
+        out = U.conv2d_NCHWc_int8(td, U.prepare_conv2d_weight(tw), s.stride, s.pad)
+        assert np.array_equal(out.cpu().numpy(), ref), U.last_variant()
+
+
+@pytest.mark.parametrize("s", WL.RESNET50, ids=lambda s: s.name)
+def test_resnet50_batch32_layer(dev, oracle, s):
+    data, wt = _layer(s, 32, 8000 + s.C + s.K)
+    ref = torch.from_numpy(oracle.c_conv2d_nchwc(data, wt, s.stride, s.pad, 1))
+    td, tw = _t(data, dev), _t(wt, dev)
+    out = U.conv2d_NCHWc_int8(td, U.prepare_conv2d_weight(tw), s.stride, s.pad)
+    assert torch.equal(out.cpu(), ref), U.last_variant()
+    del out
+    out = U.conv2d_NCHWc_int8(td, tw, s.stride, s.pad)
+    assert torch.equal(out.cpu(), ref), U.last_variant()
