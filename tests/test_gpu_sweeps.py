@@ -47,3 +47,24 @@ def test_resnet50_batch32_layer(dev, oracle, s):
     del out
     out = U.conv2d_NCHWc_int8(td, tw, s.stride, s.pad)
     assert torch.equal(out.cpu(), ref), U.last_variant()
+
+
+@pytest.mark.parametrize("s", WL.RESNET50, ids=lambda s: s.name)
+def test_resnet50_batch32_layer_fused_requantised_and_nchw(dev, oracle, s):
+    """The same layers in the fused signed form (bias, scale 11: apps/cpu/relay/result.log:3-26), with the NCHW store,
+    and requantised to u8, each against the oracle's operator built on the VNNI convolution."""
+    data, wt = _layer(s, 32, 9000 + s.C + s.K)
+    data_s8 = data.view(np.int8)
+    bias = (rng.uniform_s8((s.K,), 9100 + s.K).astype(np.int32) * 1000)
+    ref = oracle.conv2d_nchwc_int8_fused(data_s8, wt, bias, 11, s.stride, s.pad, 1, conv=oracle.c_conv2d_nchwc)
+    td, tb = _t(data_s8, dev), _t(bias, dev)
+    wp = U.prepare_conv2d_weight(_t(wt, dev))
+    out = U.conv2d_NCHWc_int8_fused(td, wp, tb, 11, s.stride, s.pad)
+    assert torch.equal(out.cpu(), torch.from_numpy(ref)), U.last_variant()
+    del out
+    planar = U.conv2d_NCHWc_int8_fused(td, wp, tb, 11, s.stride, s.pad, out_layout="NCHW")
+    assert torch.equal(planar.cpu(), torch.from_numpy(oracle.unpack_nchwc(ref))), U.last_variant()
+    del planar, ref
+    q_ref = oracle.conv2d_nchwc_u8_requant(data, wt, bias, 3, 16, s.stride, s.pad, 1, conv=oracle.c_conv2d_nchwc)
+    q = U.conv2d_NCHWc_int8_requant(_t(data, dev), wp, tb, 3, 16, s.stride, s.pad)
+    assert torch.equal(q.cpu(), torch.from_numpy(q_ref)), U.last_variant()
