@@ -68,3 +68,26 @@ def test_resnet50_batch32_layer_fused_requantised_and_nchw(dev, oracle, s):
     q_ref = oracle.conv2d_nchwc_u8_requant(data, wt, bias, 3, 16, s.stride, s.pad, 1, conv=oracle.c_conv2d_nchwc)
     q = U.conv2d_NCHWc_int8_requant(_t(data, dev), wp, tb, 3, 16, s.stride, s.pad)
     assert torch.equal(q.cpu(), torch.from_numpy(q_ref)), U.last_variant()
+
+
+REL_TOL = 1e-2  # the tolerance BASELINE states for fp16 (max relative error against float64 on the fp16-rounded inputs)
+
+
+def _max_rel(got, ref):
+    return float((np.abs(got - ref) / np.maximum(np.abs(ref), 1e-3 * np.abs(ref).max())).max())
+
+
+@pytest.mark.parametrize("s", [s for s in WL.RESNET50 if s.C % 16 == 0], ids=lambda s: s.name)
+def test_resnet50_batch32_layer_fp16(dev, oracle, s):
+    """fp16 variant of the sweep: valid convolution on the pre-padded input (the operator has no padding argument,
+    python/tensorizer/ops/gpu.py:8-53), reference layout and prepared weights, against float64."""
+    hp, wp = s.H + 2 * s.pad, s.W + 2 * s.pad
+    a = rng.normal_f16((32, s.C // 16, hp, wp, 16), 9500 + s.C + s.K)
+    b = rng.normal_f16((s.K // 16, s.C // 16, s.KH, s.KW, 16, 16), 9600 + s.K, 1.0 / np.sqrt(s.C * s.KH * s.KW))
+    ref = oracle.conv2d_nchw16c_f16(a, b, s.stride, s.stride)
+    ta, tb = _t(a, dev), _t(b, dev)
+    out = U.conv2d_NCHW16c_OHWI16o(ta, tb, s.stride, s.stride, "float32")
+    assert tuple(out.shape) == ref.shape
+    assert _max_rel(out.cpu().numpy(), ref) <= REL_TOL, U.last_variant()
+    prepared = U.conv2d_NCHW16c_OHWI16o(ta, U.prepare_conv2d_weight(tb), s.stride, s.stride, "float32")
+    assert _max_rel(prepared.cpu().numpy(), ref) <= REL_TOL, U.last_variant()
