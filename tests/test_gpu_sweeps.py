@@ -91,3 +91,15 @@ def test_resnet50_batch32_layer_fp16(dev, oracle, s):
     assert _max_rel(out.cpu().numpy(), ref) <= REL_TOL, U.last_variant()
     prepared = U.conv2d_NCHW16c_OHWI16o(ta, U.prepare_conv2d_weight(tb), s.stride, s.stride, "float32")
     assert _max_rel(prepared.cpu().numpy(), ref) <= REL_TOL, U.last_variant()
+
+
+def test_int8_gemm_4096_cubed_bit_exact(dev, oracle):
+    """BASELINE config 1 at full size against the VNNI oracle: un-packed and pre-packed weights, every element."""
+    M = N = K = 4096
+    a = rng.uniform_u8((M, K), 9701)
+    w = rng.uniform_s8((N, K), 9702)
+    wp = oracle.prepack_dense_weight(w)
+    ref = torch.from_numpy(oracle.c_dense(a, wp))
+    ta = _t(a, dev)
+    assert torch.equal(U.dense(ta, _t(w, dev)).cpu(), ref), U.last_variant()
+    assert torch.equal(U.dense_dotprod(ta, _t(wp, dev)).cpu(), ref), U.last_variant()
