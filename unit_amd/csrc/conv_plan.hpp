@@ -53,9 +53,20 @@ inline ConvPlan heuristic_plan(int npix, int K, int kbytes, bool allow_split, bo
     // thousand waves on the chip; the smallest problems use 64 x 32 (fp16: 32 x 64) tiles.
     const long t64 = tiles(64, 64);
     int v;
-    if (allow_split)  // the int8 operator
-      v = t64 >= 512 ? 64 : (t64 >= 256 ? 63 : (t64 >= 96 ? 53 : 60));
-    else
+    if (allow_split) {  // the int8 operator; distilled from the tuner's choices on cold operands (batch 1 .. 128)
+      const int nsteps = kbytes / 32;
+      const bool wide = K % 128 == 0;  // 128-channel tiles
+      if (t64 < 196)
+        v = 60;  // 64 x 32 tiles, four k-groups, six deep
+      else if (t64 < 392)
+        v = nsteps >= 36 ? 63 : 52;  // 64 x 64, four k-groups: six deep for long reductions, else four
+      else if (t64 < 784)
+        v = nsteps <= 4 ? 70 : (nsteps <= 8 ? 50 : (nsteps < 72 || !wide ? 52 : 56));
+      else if (t64 < 1568)
+        v = nsteps <= 4 ? 70 : (nsteps <= 16 ? 71 : 68);  // one wave per tile: 2 / 3 deep at four waves per SIMD, then 6 deep
+      else
+        v = nsteps <= 8 ? 70 : (nsteps >= 32 && wide ? 54 : 71);
+    } else
       v = t64 >= 512 ? 65 : (t64 >= 96 ? 63 : 61);
     return ConvPlan{v, 1, 0};
   }
