@@ -66,8 +66,20 @@ inline ConvPlan heuristic_plan(int npix, int K, int kbytes, bool allow_split, bo
         v = nsteps <= 4 ? 70 : (nsteps <= 16 ? 71 : 68);  // one wave per tile: 2 / 3 deep at four waves per SIMD, then 6 deep
       else
         v = nsteps <= 8 ? 70 : (nsteps >= 32 && wide ? 54 : 71);
-    } else
-      v = t64 >= 512 ? 65 : (t64 >= 96 ? 63 : 61);
+    } else {  // the fp16 operator (a k-step is one tap of 16 channels), same source
+      const int nsteps = kbytes / 32;
+      const bool wide = K % 128 == 0;
+      if (t64 < 196)
+        v = 60;
+      else if (t64 < 392)
+        v = nsteps <= 8 ? 50 : 52;
+      else if (t64 < 784)
+        v = nsteps <= 8 ? 50 : (nsteps <= 36 || !wide ? 68 : 56);
+      else if (t64 < 1568)
+        v = nsteps <= 8 ? 65 : (!wide ? 68 : (nsteps <= 36 ? 54 : 55));
+      else
+        v = nsteps <= 8 ? 50 : (wide ? 54 : 68);
+    }
     return ConvPlan{v, 1, 0};
   }
   int v;
