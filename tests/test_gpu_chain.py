@@ -73,8 +73,10 @@ def test_chain_graph_replay_follows_the_input(dev, oracle):
         assert np.array_equal(got, _oracle_chain(oracle, layers_np, x)[-1])
 
 
-def test_resnet50_chain_batch1_bit_exact(dev, oracle):
-    """All 52 layers at batch 1.  The oracle runs first, layer by layer, and picks each layer's shift from its own
+@pytest.mark.parametrize("builder,count,last_shape", [(chain.resnet50_layers, 52, (1, 128, 7, 7, 16)),
+                                                      (chain.resnet18_layers, 19, (1, 32, 7, 7, 16))])
+def test_resnet_chain_batch1_bit_exact(dev, oracle, builder, count, last_shape):
+    """Every layer at batch 1.  The oracle runs first, layer by layer, and picks each layer's shift from its own
     int32 sums (95th percentile -> about 200) so that the activations stay spread over 0..255 down the chain."""
     weights = []
 
@@ -82,8 +84,8 @@ def test_resnet50_chain_batch1_bit_exact(dev, oracle):
         weights.append(rng.uniform_s8((oc, ic, k, k), 1000 + len(weights)))
         return _t(weights[-1], dev)
 
-    layers = chain.resnet50_layers(make_weight)
-    assert len(layers) == 52
+    layers = builder(make_weight)
+    assert len(layers) == count
     x = rng.uniform_u8((1, 4, 56, 56, 16), 5)
     want = []
     for i, ly in enumerate(layers):
@@ -100,7 +102,7 @@ def test_resnet50_chain_batch1_bit_exact(dev, oracle):
     for i, w in enumerate(want):
         assert np.array_equal(c.outputs[i].cpu().numpy(), w), f"layer {i} ({c.variants[i]})"
         assert (w > 0).mean() > 0.2 and w.max() > 100, f"layer {i}: degenerate activations"
-    assert tuple(c.outputs[-1].shape) == (1, 128, 7, 7, 16)
+    assert tuple(c.outputs[-1].shape) == last_shape
 
 
 def test_chain_rejects_mismatched_layers(dev):

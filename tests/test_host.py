@@ -97,6 +97,23 @@ def test_resnet50_chain_lists_the_logged_shapes():
     assert seen == want
 
 
+def test_resnet18_chain_lists_the_logged_shapes():
+    from collections import Counter
+    from unit_amd import chain
+    layers = chain.resnet18_layers(lambda oc, ic, k: (oc, ic, k))
+    assert len(layers) == 19
+    hw, seen = {-1: 56}, Counter()
+    for i, ly in enumerate(layers):
+        assert -1 <= ly.source < i
+        oc, ic, k = ly.weight
+        seen[(ic, hw[ly.source], oc, k, ly.stride, ly.padding)] += 1
+        hw[i] = (hw[ly.source] + 2 * ly.padding - k) // ly.stride + 1
+        if ly.source >= 0:
+            assert layers[ly.source].weight[0] == ic
+    want = Counter({(s.C, s.H, s.K, s.KH, s.stride, s.pad): s.count for s in WL.RESNET18[1:]})
+    assert seen == want
+
+
 def test_tuned_tables_name_existing_variants():
     """Every row of the tuned tables compiled into the library names a kernel variant that exists; the tables for
     prepared weights only name direct variants (the only ones that read the prepared layout)."""

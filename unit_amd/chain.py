@@ -142,3 +142,27 @@ def resnet50_layers(make_weight, make_bias=None, scale=3, shift=14):
                 add(4 * mid, c_in, 1, stride, 0, block_in)  # projection shortcut
             block_in, c_in = last, 4 * mid
     return layers
+
+
+def resnet18_layers(make_weight, make_bias=None, scale=3, shift=14):
+    """The 19 convolutions of ResNet-18 v1 behind the stem and its pooling (cpu-shapes.log:368-386: 8 basic blocks of
+    two 3x3 convolutions in stages of 2, 2, 2, 2; a stage's first block has stride 2 on its first 3x3 and a 1x1
+    stride-2 projection shortcut, taken here as a side branch on the block's input).  Residual additions are
+    left out as in resnet50_layers.  Input of the chain: (N, 4, 56, 56, 16) u8 (64 channels)."""
+    layers = []
+    block_in, c_in = -1, 64
+
+    def add(oc, ic, k, stride, pad, source):
+        layers.append(ChainLayer(make_weight(oc, ic, k), make_bias(oc) if make_bias else None, scale, shift, stride, pad,
+                                 source))
+        return len(layers) - 1
+
+    for stage, width in enumerate((64, 128, 256, 512)):
+        for b in range(2):
+            stride = 2 if (b == 0 and stage > 0) else 1
+            a = add(width, c_in, 3, stride, 1, block_in)
+            last = add(width, width, 3, 1, 1, a)
+            if stride == 2:
+                add(width, c_in, 1, 2, 0, block_in)  # projection shortcut
+            block_in, c_in = last, width
+    return layers
