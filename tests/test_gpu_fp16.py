@@ -34,7 +34,9 @@ def test_mfma_tile_f16_lane_layout(dev):
     assert np.array_equal(tc.cpu().numpy(), (a.astype(np.float64) @ b.astype(np.float64).T).astype(np.float32))
 
 
-GEMM_CASES = [(128, 768, 3072), (32, 32, 64), (100, 132, 72), (512, 4096, 256), (4096, 2048, 512), (2050, 4100, 136)]
+GEMM_CASES = [(128, 768, 3072), (32, 32, 64), (100, 132, 72), (512, 4096, 256), (4096, 2048, 512), (2050, 4100, 136),
+              (1024, 4096, 128), (1000, 4100, 192),  # 256 x 128 tiles of the hybrid pipeline, whole and ragged
+              (2050, 4100, 192)]                     # 256 x 256 tiles, ragged
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_CASES)

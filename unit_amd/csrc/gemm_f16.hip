@@ -128,12 +128,24 @@ int gemm_f16(const void *a, const void *b, void *c, int M, int N, int K, hipStre
     case 6: return run_gemm_f16<Tile<128, 256, 128, 4, 2>, OUT_F16>(a, b, c, M, N, K, s);
     case 7: if (K % 64 == 0 && K >= 128) return run_gemm_f16_hybrid<Tile<256, 256, 128, 4, 2>, OUT_F16>(a, b, c, M, N, K, s); break;
     case 8: if (K % 64 == 0 && K >= 128) return run_gemm_f16_hybrid<Tile<256, 256, 128, 2, 4>, OUT_F16>(a, b, c, M, N, K, s); break;
+    case 9: if (K % 64 == 0 && K >= 128) return run_gemm_f16_hybrid<Tile<256, 128, 128, 2, 2>, OUT_F16>(a, b, c, M, N, K, s); break;
     default: break;
   }
+  // K a whole number of 128-byte stages: a straight into LDS, b through the transposing register loader
+  // (measured 130 us against 154 us for the all-register pipeline at 4096^3, same bits).  256 x 256 tiles of eight
+  // waves, or 256 x 128 tiles of four when those need fewer rounds of 256 workgroups for their cost (about 0.55 of
+  // a 256 x 256 tile: 2048^3 54 -> 36 us, 1024 x 4096 x 4096 95 -> 63 us, 8192 x 1024 x 1024 31 -> 25 us;
+  // 3072^3 stays on 144 large tiles, 76 us, against 106 us on 288 small ones)
+  if (M >= 256 && N >= 128 && K % 64 == 0 && K >= 128) {
+    const long tiles_half = (long)ceil_div(M, 256) * ceil_div(N, 128);
+    const long rounds_big = ceil_div((int)tiles_big, 256), rounds_half = ceil_div((int)tiles_half, 256);
+    const bool big_ok = N >= 256 && tiles_big >= 128;
+    if (big_ok && rounds_big * 100 <= rounds_half * 55)
+      return run_gemm_f16_hybrid<Tile<256, 256, 128, 2, 4>, OUT_F16>(a, b, c, M, N, K, s);
+    if (tiles_half >= 128) return run_gemm_f16_hybrid<Tile<256, 128, 128, 2, 2>, OUT_F16>(a, b, c, M, N, K, s);
+    if (big_ok) return run_gemm_f16_hybrid<Tile<256, 256, 128, 2, 4>, OUT_F16>(a, b, c, M, N, K, s);
+  }
   if (M >= 256 && N >= 256 && tiles_big >= 128) {
-    // K a whole number of 128-byte stages: a straight into LDS, b through the transposing register loader
-    // (measured 130 us against 154 us for the all-register pipeline at 4096^3, same bits)
-    if (K % 64 == 0 && K >= 128) return run_gemm_f16_hybrid<Tile<256, 256, 128, 2, 4>, OUT_F16>(a, b, c, M, N, K, s);
     // 64 (m) x 128 (n) wave tiles: measured 8-10 % faster than 128 x 64 (512-byte row runs per wave in the write-back)
     return run_gemm_f16<Tile<256, 256, 128, 4, 2>, OUT_F16>(a, b, c, M, N, K, s);
   }
