@@ -68,7 +68,8 @@ def test_gemm_fp16_k_splits(dev, oracle, M, N, K):
         assert U.last_variant().endswith("_s1") and max_rel(half.cpu().numpy(), ref) <= REL_TOL
 
 
-PREPARED_GEMM_CASES = GEMM_CASES + [(4096, 4096, 1024), (2304, 2560, 192), (257, 260, 64), (3000, 2052, 200)]
+PREPARED_GEMM_CASES = GEMM_CASES + [(4096, 4096, 1024), (2304, 2560, 192), (257, 260, 64), (3000, 2052, 200),
+                                    (2048, 2048, 320)]  # 256 x 128 tiles: a direct to LDS, prepared b through registers
 
 
 @pytest.mark.parametrize("M,N,K", PREPARED_GEMM_CASES)
@@ -93,14 +94,14 @@ def test_gemm_fp16_prepared_b(dev, oracle, M, N, K, out_dtype):
 
 
 def test_gemm_fp16_prepared_b_integer_exact(dev, oracle):
-    M, N, K = 512, 768, 1024   # large enough for the direct-to-LDS kernel (256 x 256 tiles, K % 64 == 0)
+    M, N, K = 512, 768, 1024
     a = (np.arange(M * K).reshape(M, K) % 7).astype(np.float16)
     b = (np.arange(K * N).reshape(K, N) % 5 - 2).astype(np.float16)
-    for m, n in ((M, N), (4096, 2048)):
+    for (m, n), kernel in (((M, N), "f16gemmbt_x"), ((4096, 2048), "hybrid_x256_y128"), ((4096, 4096), "dma_x256_y256")):
         aa = np.resize(a, (m, K)); bb = np.resize(b, (K, n))
         out = U.gemm_fp16(_t(aa, dev), U.prepare_gemm_b(_t(bb, dev))).cpu().numpy()
         assert np.array_equal(out.astype(np.float64), oracle.gemm_f16(aa, bb)), U.last_variant()
-    assert "dma" in U.last_variant()
+        assert kernel in U.last_variant(), U.last_variant()  # registers; 256 x 128 hybrid; 256 x 256 all direct-to-LDS
 
 
 def test_gemm_fp16_integer_exact(dev, oracle):

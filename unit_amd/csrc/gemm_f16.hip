@@ -58,6 +58,31 @@ int run_gemm_f16_hybrid(const void *a, const void *b, void *c, int M, int N, int
   return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "unit_gemm_f16: launch: %s", hipGetErrorString(e));
 }
 
+// prepared b (N, K) with a straight into LDS and b through the (non-transposing) register loader: the tile shapes the
+// all-direct kernel cannot carry (too few MFMAs per k-step for its waits)
+template <class T, bool OUT_F16>
+int run_gemm_f16_bt_hybrid(const void *a, const void *bt, void *c, int M, int N, int K, hipStream_t s) {
+  using YL = RowMajorLoader<T::BY, T::BKB, T::NT, false, 1, false>;
+  using Epi = GemmEpilogue<OpF16, OUT_F16>;
+  DmaParams p{static_cast<const char *>(a), nullptr, M, N, K * 2};
+  typename YL::Params yp{static_cast<const char *>(bt), N, K * 2, K * 2};
+  typename Epi::Params ep{c, M, N};
+  const int nk = K * 2 / T::BKB, gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
+  constexpr int lds = 2 * T::STAGE;
+  auto kern = mma_hybrid_kernel<OpF16, T, YL, Epi>;
+  static thread_local bool allowed = false;
+  if (!allowed) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
+    if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "unit_gemm_f16_prepared: hipFuncSetAttribute: %s", hipGetErrorString(e));
+    allowed = true;
+  }
+  GridMap gm{gx, gy, gx < 4 ? gx : 4, 1, gx * gy};
+  set_variant("f16gemmbt_hybrid_x%d_y%d_k%d_w%dx%d%s", T::BX, T::BY, T::BKB, T::WX, T::WY, OUT_F16 ? "_h" : "");
+  hipLaunchKernelGGL(kern, dim3(gm.total), dim3(T::NT), lds, s, p, yp, ep, nk, gm);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "unit_gemm_f16_prepared: launch: %s", hipGetErrorString(e));
+}
+
 // the same operands through registers (any K that is a multiple of 8; small problems)
 template <class T, bool OUT_F16>
 int run_gemm_f16_bt(const void *a, const void *bt, void *c, int M, int N, int K, hipStream_t s) {
@@ -77,10 +102,16 @@ int run_gemm_f16_bt(const void *a, const void *bt, void *c, int M, int N, int K,
 template <bool OUT_F16>
 int gemm_f16_bt(const void *a, const void *bt, void *c, int M, int N, int K, hipStream_t s) {
   const long tiles_big = (long)ceil_div(M, 256) * ceil_div(N, 256);
-  if (M >= 256 && N >= 256 && tiles_big >= 128) {
-    if (K % 64 == 0 && K >= 128) return run_gemm_f16_bt_dma<Tile<256, 256, 128, 2, 4>, 2, OUT_F16>(a, bt, c, M, N, K, s);
-    return run_gemm_f16_bt<Tile<256, 256, 128, 2, 4>, OUT_F16>(a, bt, c, M, N, K, s);
+  if (M >= 256 && N >= 128 && K % 64 == 0 && K >= 128) {  // tile choice as in gemm_f16 below
+    const long tiles_half = (long)ceil_div(M, 256) * ceil_div(N, 128);
+    const long rounds_big = ceil_div((int)tiles_big, 256), rounds_half = ceil_div((int)tiles_half, 256);
+    const bool big_ok = N >= 256 && tiles_big >= 128;
+    if (big_ok && rounds_big * 100 <= rounds_half * 55)
+      return run_gemm_f16_bt_dma<Tile<256, 256, 128, 2, 4>, 2, OUT_F16>(a, bt, c, M, N, K, s);
+    if (tiles_half >= 128) return run_gemm_f16_bt_hybrid<Tile<256, 128, 128, 2, 2>, OUT_F16>(a, bt, c, M, N, K, s);
+    if (big_ok) return run_gemm_f16_bt_dma<Tile<256, 256, 128, 2, 4>, 2, OUT_F16>(a, bt, c, M, N, K, s);
   }
+  if (M >= 256 && N >= 256 && tiles_big >= 128) return run_gemm_f16_bt<Tile<256, 256, 128, 2, 4>, OUT_F16>(a, bt, c, M, N, K, s);
   return run_gemm_f16_bt<Tile<128, 128, 64, 2, 2>, OUT_F16>(a, bt, c, M, N, K, s);
 }
 

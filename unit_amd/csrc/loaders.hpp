@@ -26,6 +26,7 @@ struct RowMajorLoader {
   static constexpr bool kNeedsSync = false;
   static constexpr int kPF = PF;
   static constexpr int CPR = BKB / 16, RPP = NT / CPR, NCH = ROWS / RPP;
+  static constexpr int kLoads = NCH;  // global loads per thread and stage
   static_assert(NT % CPR == 0 && ROWS % RPP == 0 && RPP % 16 == 0, "row-major loader shape");
 
   v4i r[PF][NCH];
