@@ -71,13 +71,13 @@ def main():
     def dev_t(a):
         return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
 
-    def time_us(fn, iters, warm=3, bursts=1):
+    def time_us(fn, iters, warm=3, bursts=1, median=False):
         """Mean launch-to-launch time of `iters` back-to-back launches; with bursts > 1 the fastest burst (the
-        clocks of this part follow the load of whatever ran just before)."""
+        clocks of this part follow the load of whatever ran just before), or the median one."""
         for _ in range(warm):
             fn()
         torch.cuda.synchronize()
-        best = float("inf")
+        seen = []
         for _ in range(bursts):
             s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             s.record()
@@ -85,8 +85,8 @@ def main():
                 fn()
             e.record()
             torch.cuda.synchronize()
-            best = min(best, s.elapsed_time(e) * 1e3 / iters)
-        return best
+            seen.append(s.elapsed_time(e) * 1e3 / iters)
+        return sorted(seen)[len(seen) // 2] if median else min(seen)
 
     if args.profile in ("gemm_i8", "gemm_f16", "gemm_f16_prepared", "copy"):
         n = 4096
@@ -219,11 +219,12 @@ def main():
         ref_weights = dict(workload="the same step with every convolution on the reference's blocked weight layout",
                            ms_per_step=round(ref_ms, 4), tops=round(step_ops / (ref_ms * 1e-3) / 1e12, 2))
 
-    # per-layer launch duration (HIP events on the launch stream, back-to-back launches)
+    # per-layer launch duration (HIP events on the launch stream, back-to-back launches; the median of three bursts of
+    # 30 launches: a single burst now and then lands 20 % high on the write-bound layers)
     ridge = PEAK_INT8_TOPS * 1e12 / (PEAK_HBM_GBS * 1e9)
     table = []
     for ly in layers:
-        us = time_us(ly["call"], 30)
+        us = time_us(ly["call"], 30, bursts=3, median=True)
         ai = ly["ops"] / ly["bytes"]
         bound = "mfma" if ai >= ridge else "hbm"
         tops, gbs = ly["ops"] / us / 1e6, ly["bytes"] / us / 1e3
