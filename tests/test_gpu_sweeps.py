@@ -103,3 +103,35 @@ def test_int8_gemm_4096_cubed_bit_exact(dev, oracle):
     ta = _t(a, dev)
     assert torch.equal(U.dense(ta, _t(w, dev)).cpu(), ref), U.last_variant()
     assert torch.equal(U.dense_dotprod(ta, _t(wp, dev)).cpu(), ref), U.last_variant()
+
+
+def _random_mid_cases(count, seed):
+    r = np.random.RandomState(seed)
+    cases = []
+    for _ in range(count):
+        ks = int(r.choice([1, 1, 3]))
+        cases.append((int(r.choice([1, 2, 4, 8, 16])), 16 * int(r.randint(1, 33)), int(r.randint(7, 41)), int(r.randint(7, 41)),
+                      16 * int(r.randint(1, 33)), ks, int(r.choice([1, 1, 2])), ks // 2))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_mid_cases(24, 20250101), ids=lambda c: "x".join(str(v) for v in c))
+def test_heuristic_choices_on_random_mid_size_layers(dev, oracle, monkeypatch, case):
+    """Shapes outside the tuned tables (the tables are switched off): whatever variant the heuristic picks, the int8
+    result is bit-exact on both weight layouts and the fp16 one within tolerance."""
+    monkeypatch.setenv("UNIT_AMD_CONV_NOTABLE", "1")
+    n, c, h, w, k, ks, stride, pad = case
+    data = rng.uniform_u8((n, c // 16, h, w, 16), 9800 + c)
+    wt = rng.uniform_s8((k // 16, c // 16, ks, ks, 4, 16, 4), 9801 + k)
+    ref = oracle.c_conv2d_nchwc(data, wt, stride, pad, 1)
+    td, tw = _t(data, dev), _t(wt, dev)
+    assert np.array_equal(U.conv2d_NCHWc_int8(td, tw, stride, pad).cpu().numpy(), ref), U.last_variant()
+    out = U.conv2d_NCHWc_int8(td, U.prepare_conv2d_weight(tw), stride, pad)
+    assert np.array_equal(out.cpu().numpy(), ref), U.last_variant()
+    if n <= 4:  # the float64 oracle is numpy
+        hp, wp = h + 2 * pad, w + 2 * pad
+        a = rng.normal_f16((n, c // 16, hp, wp, 16), 9802 + c)
+        b = rng.normal_f16((k // 16, c // 16, ks, ks, 16, 16), 9803 + k, 1.0 / np.sqrt(c * ks * ks))
+        fref = oracle.conv2d_nchw16c_f16(a, b, stride, stride)
+        got = U.conv2d_NCHW16c_OHWI16o(_t(a, dev), U.prepare_conv2d_weight(_t(b, dev)), stride, stride, "float32")
+        assert _max_rel(got.cpu().numpy(), fref) <= REL_TOL, U.last_variant()
