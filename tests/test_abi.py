@@ -122,8 +122,11 @@ def test_out_hw_and_error_paths_without_gpu():
     assert L.unit_gemm_f16_prepared(16, 16, 16, 16, 6, 16, 0, None) == -1 and b"multiple of 4" in L.unit_last_error()
     assert L.unit_gemm_f16_prepared(16, None, 16, 16, 8, 16, 0, None) == -1 and b"null" in L.unit_last_error()
     assert L.unit_gemm_f16_prepared(16, 8, 16, 16, 8, 16, 0, None) == -1 and b"aligned" in L.unit_last_error()
-    # size limit: every tensor must stay below 2^31 bytes (32-bit offsets in the kernels)
-    huge = _lib.ConvDesc(4096, 256, 56, 56, 256, 1, 1, 1, 1, 0, 0, 0, 0, 1, 1, 16)
+    # size limit: weights, GEMM operands and a single image of a convolution stay below 2^31 bytes (32-bit
+    # offsets in the kernels); a larger batch is sliced instead and reaches the pointer checks
+    huge = _lib.ConvDesc(2, 256, 4096, 4096, 256, 1, 1, 1, 1, 0, 0, 0, 0, 1, 1, 16)
+    many = _lib.ConvDesc(4096, 256, 56, 56, 256, 1, 1, 1, 1, 0, 0, 0, 0, 1, 1, 16)
+    assert L.unit_conv2d_nchwc_u8s8s32(ctypes.byref(many), 1, 1, 1, None) == -1 and b"aligned" in L.unit_last_error()
     assert L.unit_conv2d_nchwc_u8s8s32(ctypes.byref(huge), 1, 1, 1, None) == -1 and b"2^31" in L.unit_last_error()
     assert L.unit_dense_u8s8s32(1, 1, 1, 65536, 65536, 16, None) == -1 and b"2^31" in L.unit_last_error()
     with pytest.raises(ValueError):

@@ -68,6 +68,11 @@ extern "C" int unit_conv2d_nchw16c_f16f32(const unit_conv_desc *d, const void *a
   if (d->cb != 16) return fail(UNIT_E_ARG, "%s: cb must be 16 (got %d)", what, d->cb);
   if (d->pt || d->pl || d->pb || d->pr) return fail(UNIT_E_ARG, "%s: the operator has no padding argument; pre-pad the data", what);
   if (d->dh != 1 || d->dw != 1) return fail(UNIT_E_ARG, "%s: dilation must be 1", what);
+  size_t in_img, out_img;
+  if (const int per = batch_slice(d, (size_t)d->C * 2, (size_t)d->K * 4, &in_img, &out_img))
+    return run_batch_slices(d, per, in_img, out_img, a, out, [&](const unit_conv_desc *sd, const void *x, void *y) {
+      return unit_conv2d_nchw16c_f16f32(sd, x, b, y, stream);
+    });
   ConvGeom g;
   if (int rc = conv_geom(d, 32, &g, what)) return rc;
   if (!fits((size_t)g.npix * d->K * 4)) return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);

@@ -42,6 +42,11 @@ extern "C" int unit_conv2d_nchwc_u8s8s32(const unit_conv_desc *d, const void *da
   const char *what = "unit_conv2d_nchwc_u8s8s32";
   if (!d || !data || !weight || !out) return fail(UNIT_E_ARG, "%s: null pointer", what);
   if (d->cb != 16 && d->cb != 4) return fail(UNIT_E_ARG, "%s: cb must be 16 or 4 (got %d)", what, d->cb);
+  size_t in_img, out_img;
+  if (const int per = batch_slice(d, (size_t)d->C, (size_t)d->K * 4, &in_img, &out_img))
+    return run_batch_slices(d, per, in_img, out_img, data, out, [&](const unit_conv_desc *sd, const void *x, void *y) {
+      return unit_conv2d_nchwc_u8s8s32(sd, x, weight, y, stream);
+    });
   ConvGeom g;
   if (int rc = conv_geom(d, d->cb, &g, what)) return rc;
   if (!fits((size_t)g.npix * d->K * 4)) return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);

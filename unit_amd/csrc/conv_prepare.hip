@@ -186,6 +186,11 @@ extern "C" int unit_conv2d_nchwc_u8s8s32_prepared(const unit_conv_desc *d, const
   using namespace unit;
   const char *what = "unit_conv2d_nchwc_u8s8s32_prepared";
   if (!d || !data || !prepared || !out) return fail(UNIT_E_ARG, "%s: null pointer", what);
+  size_t in_img, out_img;
+  if (const int per = batch_slice(d, (size_t)d->C, (size_t)d->K * 4, &in_img, &out_img))
+    return run_batch_slices(d, per, in_img, out_img, data, out, [&](const unit_conv_desc *sd, const void *x, void *y) {
+      return unit_conv2d_nchwc_u8s8s32_prepared(sd, x, prepared, y, stream);
+    });
   ConvGeom g;
   if (int rc = check_prepared_conv(what, d, 16, &g, data, prepared, out)) return rc;
   const PreparedLayout pl = prepared_layout(d->K, d->C, d->KH, d->KW, d->cb, 1);
@@ -205,6 +210,11 @@ extern "C" int unit_conv2d_nchwc_u8s8u8_requant_prepared(const unit_conv_desc *d
   const char *what = "unit_conv2d_nchwc_u8s8u8_requant_prepared";
   if (!d || !data || !prepared || !out) return fail(UNIT_E_ARG, "%s: null pointer", what);
   if (shift < 1 || shift > 62) return fail(UNIT_E_ARG, "%s: shift must be in 1..62 (got %d)", what, shift);
+  size_t in_img, out_img;
+  if (const int per = batch_slice(d, (size_t)d->C, (size_t)d->K, &in_img, &out_img))
+    return run_batch_slices(d, per, in_img, out_img, data, out, [&](const unit_conv_desc *sd, const void *x, void *y) {
+      return unit_conv2d_nchwc_u8s8u8_requant_prepared(sd, x, prepared, bias, scale, shift, y, stream);
+    });
   ConvGeom g;
   if (int rc = check_prepared_conv(what, d, 16, &g, data, prepared, out)) return rc;
   const PreparedLayout pl = prepared_layout(d->K, d->C, d->KH, d->KW, d->cb, 1);
@@ -228,6 +238,13 @@ namespace {
 int fused_prepared(const char *what, const unit_conv_desc *d, const void *data, const void *prepared,
                    const int32_t *bias, int32_t scale, void *out, int planar, unit_stream_t stream) {
   if (!d || !data || !prepared || !out) return fail(UNIT_E_ARG, "%s: null pointer", what);
+  size_t in_img, out_img;
+  if (const int per = batch_slice(d, (size_t)d->C, (size_t)d->K * 4, &in_img, &out_img)) {
+    if (planar) out_img = out_img / d->K * planar;  // sliced as the blocked result would be; an image is planar channels
+    return run_batch_slices(d, per, in_img, out_img, data, out, [&](const unit_conv_desc *sd, const void *x, void *y) {
+      return fused_prepared(what, sd, x, prepared, bias, scale, y, planar, stream);
+    });
+  }
   ConvGeom g;
   if (int rc = check_prepared_conv(what, d, 16, &g, data, prepared, out)) return rc;
   const int ntable = (int)(sizeof(kTunedI8Prepared) / sizeof(kTunedI8Prepared[0])) - 1;
@@ -263,6 +280,11 @@ extern "C" int unit_conv2d_nchw16c_f16f32_prepared(const unit_conv_desc *d, cons
   if (!d || !a || !prepared || !out) return fail(UNIT_E_ARG, "%s: null pointer", what);
   if (d->pt || d->pl || d->pb || d->pr) return fail(UNIT_E_ARG, "%s: the operator has no padding argument; pre-pad the data", what);
   if (d->dh != 1 || d->dw != 1) return fail(UNIT_E_ARG, "%s: dilation must be 1", what);
+  size_t in_img, out_img;
+  if (const int per = batch_slice(d, (size_t)d->C * 2, (size_t)d->K * 4, &in_img, &out_img))
+    return run_batch_slices(d, per, in_img, out_img, a, out, [&](const unit_conv_desc *sd, const void *x, void *y) {
+      return unit_conv2d_nchw16c_f16f32_prepared(sd, x, prepared, y, stream);
+    });
   ConvGeom g;
   if (int rc = check_prepared_conv(what, d, 32, &g, a, prepared, out)) return rc;
   const int ntable = (int)(sizeof(kTunedF16Prepared) / sizeof(kTunedF16Prepared[0])) - 1;

@@ -57,6 +57,11 @@ extern "C" int unit_conv2d_nchwc_s8s8s32_fused(const unit_conv_desc *d, const vo
   using namespace unit;
   if (!d || !data || !weight || !out) return fail(UNIT_E_ARG, "%s: null pointer", kWhat);
   if (d->cb != 16 && d->cb != 4) return fail(UNIT_E_ARG, "%s: cb must be 16 or 4 (got %d)", kWhat, d->cb);
+  size_t in_img, out_img;
+  if (const int per = batch_slice(d, (size_t)d->C, (size_t)d->K * 4, &in_img, &out_img))
+    return run_batch_slices(d, per, in_img, out_img, data, out, [&](const unit_conv_desc *sd, const void *x, void *y) {
+      return unit_conv2d_nchwc_s8s8s32_fused(sd, x, weight, bias, scale, y, stream);
+    });
   ConvGeom g;
   if (int rc = conv_geom(d, d->cb, &g, kWhat)) return rc;
   if (!fits((size_t)g.npix * d->K * 4)) return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", kWhat);

@@ -54,6 +54,34 @@ inline int check_aligned(const char *what, std::initializer_list<const void *> p
   return UNIT_OK;
 }
 
+// Images per launch for a convolution whose data or result would pass the kernels' 32-bit offsets (0: the whole
+// batch fits one launch, or a single image is already too large and the entry point's own checks reject it).
+// Images lie one after the other in the blocked and in the planar layouts alike, so such a convolution runs as
+// several launches over slices of the batch.  in_px / out_px: bytes per input / output pixel over all channels.
+inline int batch_slice(const unit_conv_desc *d, size_t in_px, size_t out_px, size_t *in_img, size_t *out_img) {
+  int32_t OH = 0, OW = 0;
+  if (d->N <= 1 || unit_conv_out_hw(d, &OH, &OW) != UNIT_OK) return 0;
+  *in_img = (size_t)d->H * d->W * in_px;
+  *out_img = (size_t)OH * OW * out_px;
+  const size_t big = *in_img > *out_img ? *in_img : *out_img;
+  if (big * d->N <= kMaxTensorBytes || big > kMaxTensorBytes) return 0;
+  return (int)(kMaxTensorBytes / big);
+}
+
+// call(desc, data, out) for each slice of `per` images; stops at the first error
+template <class F>
+int run_batch_slices(const unit_conv_desc *d, int per, size_t in_img, size_t out_img, const void *data, void *out,
+                     F call) {
+  unit_conv_desc s = *d;
+  for (int n0 = 0; n0 < d->N; n0 += per) {
+    s.N = d->N - n0 < per ? d->N - n0 : per;
+    if (int rc = call(&s, static_cast<const char *>(data) + (size_t)n0 * in_img,
+                      static_cast<char *>(out) + (size_t)n0 * out_img))
+      return rc;
+  }
+  return UNIT_OK;
+}
+
 // k-splits of a GEMM.  Few output tiles and a long reduction leave most of the chip idle (the reference's own
 // GEMM sizes, 128 x 768 x 3072 in apps/gpu/gemm.py:6 and 128 x 3072 x 768 in apps/cpu/kernel/int8-gemm.py:9, are 6
 // and 24 tiles of 128 x 128; the reference splits the reduction of the first with rfactor, gemm.py:22-40): the

@@ -198,6 +198,16 @@ int nchwc(const void *src, void *dst, int N, int C, int H, int W, int cb, int es
   if (es != 1 && es != 2 && es != 4) return fail(UNIT_E_ARG, "%s: elem_size must be 1, 2 or 4 (got %d)", what, es);
   const int cc = ceil_div(C, cb);
   const size_t hw = (size_t)H * W, total = (size_t)N * cc * hw * cb;
+  if (const size_t img = (size_t)cc * hw * cb * es; N > 1 && !fits(total * es) && fits(img)) {
+    // images lie one after the other on both sides: slices of the batch that fit 32-bit offsets
+    const int per = (int)(kMaxTensorBytes / img);
+    const size_t planar = (size_t)C * hw * es, src_img = PACK ? planar : img, dst_img = PACK ? img : planar;
+    for (int n0 = 0; n0 < N; n0 += per)
+      if (int rc = nchwc<PACK>(static_cast<const char *>(src) + n0 * src_img, static_cast<char *>(dst) + n0 * dst_img,
+                               N - n0 < per ? N - n0 : per, C, H, W, cb, es, s, what))
+        return rc;
+    return UNIT_OK;
+  }
   if (!fits(total * es)) return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
   if (int rc = check_device()) return rc;
   const char *in = static_cast<const char *>(src);
