@@ -128,7 +128,8 @@ def test_out_hw_and_error_paths_without_gpu():
     many = _lib.ConvDesc(4096, 256, 56, 56, 256, 1, 1, 1, 1, 0, 0, 0, 0, 1, 1, 16)
     assert L.unit_conv2d_nchwc_u8s8s32(ctypes.byref(many), 1, 1, 1, None) == -1 and b"aligned" in L.unit_last_error()
     assert L.unit_conv2d_nchwc_u8s8s32(ctypes.byref(huge), 1, 1, 1, None) == -1 and b"2^31" in L.unit_last_error()
-    assert L.unit_dense_u8s8s32(1, 1, 1, 65536, 65536, 16, None) == -1 and b"2^31" in L.unit_last_error()
+    assert L.unit_dense_u8s8s32(1, 1, 1, 16, 65536, 65536, None) == -1 and b"2^31" in L.unit_last_error()
+    assert L.unit_dense_u8s8s32(1, 1, 1, 65536, 65536, 16, None) == -1 and b"aligned" in L.unit_last_error()  # row slices
     with pytest.raises(ValueError):
         _lib.check(-1)
 

@@ -108,3 +108,35 @@ def test_layout_kernels_beyond_the_limit(dev, oracle):
     del packed
     for a, b in _windows(n, 256 * hw * hw):
         assert torch.equal(back[a:b], x[a:b]), (a, b)
+
+
+def _row_windows(m, row_bytes):
+    per = LIMIT // row_bytes // 256 * 256  # slices are whole tiles of 256 rows
+    assert per < m, "the case does not exceed the limit"
+    return [(0, 4), (m - 4, m)] + [(b - 4, min(b + 4, m)) for b in range(per, m, per)]
+
+
+def test_gemm_results_beyond_the_limit(dev, oracle):
+    """70000 x 8192 results (2.29 GB of int32 / fp32) from a 64-long reduction: the int8 dense on both weight layouts
+    and the fp16 GEMM on both layouts of b run as slices of rows."""
+    m, n, k = 70000, 8192, 64
+    a = _randint_u8((m, k), 4501, dev)
+    w = rng.uniform_s8((n, k), 4502)
+    spans = _row_windows(m, n * 4)
+    for out in (U.dense(a, _t(w, dev)), U.dense_dotprod(a, _t(oracle.prepack_dense_weight(w), dev))):
+        assert out.numel() * 4 > LIMIT
+        for r0, r1 in spans:
+            assert np.array_equal(out[r0:r1].cpu().numpy(), oracle.dense_logical(a[r0:r1].cpu().numpy(), w)), (r0, r1)
+        del out
+    g = torch.Generator(device=dev)
+    g.manual_seed(4503)
+    a16 = torch.randn((m, k), dtype=torch.float16, device=dev, generator=g)
+    b16 = rng.normal_f16((k, n), 4504, 1.0 / np.sqrt(k))
+    tb = _t(b16, dev)
+    for b_arg in (tb, U.prepare_gemm_b(tb)):
+        out = U.gemm_fp16(a16, b_arg)
+        for r0, r1 in spans:
+            ref = oracle.gemm_f16(a16[r0:r1].cpu().numpy(), b16)
+            rel = np.abs(out[r0:r1].cpu().numpy() - ref) / np.maximum(np.abs(ref), 1e-3 * np.abs(ref).max())
+            assert float(rel.max()) <= REL_TOL, (r0, r1, U.last_variant())
+        del out

@@ -196,6 +196,10 @@ extern "C" int unit_gemm_f16(const void *a, const void *b, void *c, int32_t M, i
   if (M <= 0 || N <= 0 || K <= 0) return fail(UNIT_E_ARG, "%s: M, N, K must be positive (got %d, %d, %d)", what, M, N, K);
   if (K % 8) return fail(UNIT_E_ARG, "%s: K must be a multiple of 8 (got %d)", what, K);
   if (N % 4) return fail(UNIT_E_ARG, "%s: N must be a multiple of 4 (got %d)", what, N);
+  if (const int per = row_slice(M, (size_t)K * 2, (size_t)N * 4))
+    return run_row_slices(M, per, (size_t)K * 2, (size_t)N * (out_f16 ? 2 : 4), a, c, [&](const void *as, void *cs, int rows) {
+      return unit_gemm_f16(as, b, cs, rows, N, K, out_f16, stream);
+    });
   if (!fits((size_t)M * K * 2) || !fits((size_t)N * K * 2) || !fits((size_t)M * N * 4))
     return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
   if (int rc = check_aligned(what, {a, b, c})) return rc;
@@ -229,6 +233,10 @@ extern "C" int unit_gemm_f16_prepared(const void *a, const void *bt, void *c, in
   if (M <= 0 || N <= 0 || K <= 0) return fail(UNIT_E_ARG, "%s: M, N, K must be positive (got %d, %d, %d)", what, M, N, K);
   if (K % 8) return fail(UNIT_E_ARG, "%s: K must be a multiple of 8 (got %d)", what, K);
   if (N % 4) return fail(UNIT_E_ARG, "%s: N must be a multiple of 4 (got %d)", what, N);
+  if (const int per = row_slice(M, (size_t)K * 2, (size_t)N * 4))
+    return run_row_slices(M, per, (size_t)K * 2, (size_t)N * (out_f16 ? 2 : 4), a, c, [&](const void *as, void *cs, int rows) {
+      return unit_gemm_f16_prepared(as, bt, cs, rows, N, K, out_f16, stream);
+    });
   if (!fits((size_t)M * K * 2) || !fits((size_t)N * K * 2) || !fits((size_t)M * N * 4))
     return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
   if (int rc = check_aligned(what, {a, bt, c})) return rc;

@@ -94,6 +94,10 @@ int dense(const void *a, const void *w, void *c, int M, int N, int K, unit_strea
   if (K % 16) return fail(UNIT_E_ARG, "%s: K must be a multiple of 16 (got %d)", what, K);
   if (PACKED && N % 128) return fail(UNIT_E_ARG, "%s: N must be a multiple of 128 (got %d)", what, N);
   if (!PACKED && N % 4) return fail(UNIT_E_ARG, "%s: N must be a multiple of 4 (got %d)", what, N);
+  if (const int per = row_slice(M, (size_t)K, (size_t)N * 4))
+    return run_row_slices(M, per, (size_t)K, (size_t)N * 4, a, c, [&](const void *as, void *cs, int rows) {
+      return dense<PACKED>(as, w, cs, rows, N, K, stream);
+    });
   if (!fits((size_t)M * K) || !fits((size_t)N * K) || !fits((size_t)M * N * 4))
     return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
   if (int rc = check_aligned(what, {a, w, c})) return rc;

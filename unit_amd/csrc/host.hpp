@@ -82,6 +82,25 @@ int run_batch_slices(const unit_conv_desc *d, int per, size_t in_img, size_t out
   return UNIT_OK;
 }
 
+// Rows per launch for a GEMM whose row-major a (M, K) or c (M, N) would pass the 32-bit offsets (0: one launch, or a
+// slice of 256 rows is already too large and the entry point rejects the call).  A multiple of 256, the tile height.
+inline int row_slice(int M, size_t a_row_bytes, size_t c_row_bytes) {
+  const size_t big = a_row_bytes > c_row_bytes ? a_row_bytes : c_row_bytes;
+  if (big * M <= kMaxTensorBytes) return 0;
+  const size_t rows = kMaxTensorBytes / big / 256 * 256;
+  return rows < (size_t)M ? (int)rows : 0;
+}
+
+// call(a, c, rows) for each slice of `per` rows; stops at the first error
+template <class F>
+int run_row_slices(int M, int per, size_t a_row_bytes, size_t c_row_bytes, const void *a, void *c, F call) {
+  for (int m0 = 0; m0 < M; m0 += per)
+    if (int rc = call(static_cast<const char *>(a) + (size_t)m0 * a_row_bytes,
+                      static_cast<char *>(c) + (size_t)m0 * c_row_bytes, M - m0 < per ? M - m0 : per))
+      return rc;
+  return UNIT_OK;
+}
+
 // k-splits of a GEMM.  Few output tiles and a long reduction leave most of the chip idle (the reference's own
 // GEMM sizes, 128 x 768 x 3072 in apps/gpu/gemm.py:6 and 128 x 3072 x 768 in apps/cpu/kernel/int8-gemm.py:9, are 6
 // and 24 tiles of 128 x 128; the reference splits the reduction of the first with rfactor, gemm.py:22-40): the
