@@ -15,7 +15,7 @@
  *     unit_last_error() returns a thread-local message;
  *   - int8 results are exact (int32 accumulation, wrapping mod 2^32 like vpdpbusd);
  *     fp16 inputs are multiplied and accumulated in fp32 on the MFMA unit;
- *   - a tensor may not exceed 2^31-1 bytes; the activations of the 2-D convolutions and of the
+ *   - a tensor may not exceed 2^31-1 bytes; the activations of the convolutions and of the
  *     layout kernels may, as long as a single image stays below: such a call runs as several
  *     launches over slices of the batch; likewise a and c of the GEMMs, over slices of rows.
  */

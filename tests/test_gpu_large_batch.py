@@ -140,3 +140,14 @@ def test_gemm_results_beyond_the_limit(dev, oracle):
             rel = np.abs(out[r0:r1].cpu().numpy() - ref) / np.maximum(np.abs(ref), 1e-3 * np.abs(ref).max())
             assert float(rel.max()) <= REL_TOL, (r0, r1, U.last_variant())
         del out
+
+
+def test_conv3d_results_beyond_the_limit(dev, oracle):
+    """conv3d 16 -> 64 channels, 2 x 2 x 2 window on 8 x 56 x 56 volumes, 420 of them: 2.28 GB of int32 results."""
+    n, c, k, dd, hw = 420, 16, 64, 8, 56
+    data = _randint_u8((n, 1, dd, hw, hw, 16), 4601, dev).view(torch.int8)
+    wt = rng.uniform_s8((k // 16, 1, 2, 2, 2, 4, 16, 4), 4602)
+    out = U.conv3d_NCDHWc_int8(data, _t(wt, dev), 1)
+    assert out.numel() * 4 > LIMIT
+    for a, b in _windows(n, 7 * 55 * 55 * k * 4):
+        assert np.array_equal(out[a:b].cpu().numpy(), oracle.conv3d_ncdhwc_int8(data[a:b].cpu().numpy(), wt, 1)), (a, b)

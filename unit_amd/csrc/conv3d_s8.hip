@@ -30,6 +30,19 @@ extern "C" int unit_conv3d_ncdhwc_s8s8s32(const unit_conv3d_desc *d, const void 
   const int cc = d->C / cb;
   const size_t img = (size_t)cc * d->D * d->H * d->W * cb, opix = (size_t)OD * OH * OW, npix = opix * d->N;
   const size_t taps = (size_t)cc * d->KD * d->KH * d->KW;
+  if (const size_t out_img = opix * d->K * 4, big = img > out_img ? img : out_img;
+      d->N > 1 && big * d->N > kMaxTensorBytes && big <= kMaxTensorBytes) {
+    // beyond the 32-bit offsets: one launch per slice of the batch (volumes lie one after the other)
+    const int per = (int)(kMaxTensorBytes / big);
+    unit_conv3d_desc sd = *d;
+    for (int n0 = 0; n0 < d->N; n0 += per) {
+      sd.N = d->N - n0 < per ? d->N - n0 : per;
+      if (int rc = unit_conv3d_ncdhwc_s8s8s32(&sd, static_cast<const char *>(data) + (size_t)n0 * img, weight,
+                                              static_cast<char *>(out) + (size_t)n0 * out_img, stream))
+        return rc;
+    }
+    return UNIT_OK;
+  }
   if (!fits(img * d->N) || npix > kMaxTensorBytes || !fits((size_t)d->K * taps * cb) || !fits(npix * d->K * 4))
     return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
   if (int rc = check_aligned(what, {data, weight, out})) return rc;
