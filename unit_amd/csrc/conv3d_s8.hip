@@ -65,7 +65,7 @@ extern "C" int unit_conv3d_ncdhwc_s8s8s32(const unit_conv3d_desc *d, const void 
   // the launcher only reads K from the 2-D descriptor; the planner keys on pixels, channels and reduction length
   unit_conv_desc d2{d->N, d->C, d->H, d->W, d->K, d->KH, d->KW, d->stride, d->stride, 0, 0, 0, 0, 1, 1, cb};
   ConvPlan p = plan_conv(&d2, g.npix, g.ntaps * cb, nullptr, 0, true, true);
-  if (!kConvTiles[p.variant].direct) p = heuristic_plan(g.npix, d->K, g.ntaps * cb, true, true);
+  if (!kConvTiles[p.variant].direct) p = heuristic_plan(g.npix, d->K, g.ntaps * cb, true, true, d->stride > 1);
   p.splits = 1;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (cb == 4) return conv_c4_direct(what, p, &d2, g, data, weight, nullptr, 1, false, out, s);

@@ -44,7 +44,7 @@ struct TunedConv {
 // layers (few input channels, many pixels) want 64..128-pixel tiles of 64 channels with many
 // workgroups in flight; long reductions want the 128-channel tiles with two stages of loads in
 // flight; the 256 x 256 tiles only pay when they still give every CU several workgroups.
-inline ConvPlan heuristic_plan(int npix, int K, int kbytes, bool allow_split, bool direct_ok) {
+inline ConvPlan heuristic_plan(int npix, int K, int kbytes, bool allow_split, bool direct_ok, bool strided = false) {
   const bool k128 = kbytes % 128 == 0;
   const auto tiles = [&](int bx, int by) { return (long)ceil_div(K, bx) * ceil_div(npix, by); };
   if (direct_ok) {
@@ -52,8 +52,8 @@ inline ConvPlan heuristic_plan(int npix, int K, int kbytes, bool allow_split, bo
     // 64 x 64 tile when the tiles alone fill the SIMDs, else k-groups (4, 8) to put about a
     // thousand waves on the chip; the smallest problems use 64 x 32 (fp16: 32 x 64) tiles.
     const long t64 = tiles(64, 64);
-    int v;
-    if (allow_split) {  // the int8 operator; distilled from the tuner's choices on cold operands (batch 1 .. 128)
+    int v, panel = 0;
+    if (allow_split) {  // the int8 operator; distilled from the tuner's choices on cold operands (batch 1 .. 256)
       const int nsteps = kbytes / 32;
       const bool wide = K % 128 == 0;  // 128-channel tiles
       if (t64 < 196)
@@ -64,8 +64,14 @@ inline ConvPlan heuristic_plan(int npix, int K, int kbytes, bool allow_split, bo
         v = nsteps <= 4 ? 70 : (nsteps <= 8 ? 50 : (nsteps < 72 || !wide ? 52 : 56));
       else if (t64 < 1568)
         v = nsteps <= 4 ? 70 : (nsteps <= 16 ? 71 : 68);  // one wave per tile: 2 / 3 deep at four waves per SIMD, then 6 deep
+      else if (t64 < 3136)
+        v = nsteps <= 8 ? 70 : (wide ? 54 : 71);  // 128-channel tiles while they still give every SIMD a wave
       else
-        v = nsteps <= 8 ? 70 : (nsteps >= 32 && wide ? 54 : 71);
+        v = nsteps <= 36 ? 70 : 68;
+      // Eight or more channel tiles: panels of four, so that an XCD's L2 holds a slice of the weights for all its
+      // pixels; not when the stride skips input pixels (the data is then the sparse operand), nor when a long
+      // reduction already keeps a large problem's weights hot.
+      if (K >= 512 && !strided && (nsteps <= 16 || t64 < 784)) panel = 4;
     } else {  // the fp16 operator (a k-step is one tap of 16 channels), same source
       const int nsteps = kbytes / 32;
       const bool wide = K % 128 == 0;
@@ -80,7 +86,7 @@ inline ConvPlan heuristic_plan(int npix, int K, int kbytes, bool allow_split, bo
       else
         v = nsteps <= 8 ? 50 : (wide ? 54 : 68);
     }
-    return ConvPlan{v, 1, 0};
+    return ConvPlan{v, 1, panel};
   }
   int v;
   if (K % 128 != 0) {  // 64-channel tiles
@@ -108,7 +114,7 @@ inline ConvPlan heuristic_plan(int npix, int K, int kbytes, bool allow_split, bo
 
 inline ConvPlan plan_conv(const unit_conv_desc *d, int npix, int kbytes, const TunedConv *table, int ntable,
                           bool allow_split, bool direct_ok) {
-  ConvPlan p = heuristic_plan(npix, d->K, kbytes, allow_split, direct_ok);
+  ConvPlan p = heuristic_plan(npix, d->K, kbytes, allow_split, direct_ok, d->sh * d->sw > 1);
   // UNIT_AMD_CONV_NOTABLE=1: heuristic only (the tuner measures it as the baseline)
   if (tuning_override("UNIT_AMD_CONV_NOTABLE") > 0) ntable = 0;
   for (int i = 0; i < ntable; ++i) {

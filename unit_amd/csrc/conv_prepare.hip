@@ -117,7 +117,7 @@ const TunedConv kTunedF16Prepared[] = {
 ConvPlan plan_prepared(const unit_conv_desc *d, const ConvGeom &g, int kbytes, const TunedConv *table, int ntable,
                        bool int8) {
   ConvPlan p = plan_conv(d, g.npix, kbytes, table, ntable, int8, true);
-  if (!kConvTiles[p.variant].direct) p = heuristic_plan(g.npix, d->K, kbytes, int8, true);
+  if (!kConvTiles[p.variant].direct) p = heuristic_plan(g.npix, d->K, kbytes, int8, true, d->sh * d->sw > 1);
   p.splits = 1;
   return p;
 }

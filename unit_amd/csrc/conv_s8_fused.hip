@@ -73,7 +73,7 @@ extern "C" int unit_conv2d_nchwc_s8s8s32_fused(const unit_conv_desc *d, const vo
     int ntable = 0;
     const TunedConv *table = tuned_conv_i8(&ntable);
     ConvPlan p = plan_conv(d, g.npix, g.ntaps * d->cb, table, ntable, true, true);
-    if (!kConvTiles[p.variant].direct) p = heuristic_plan(g.npix, d->K, g.ntaps * d->cb, true, true);
+    if (!kConvTiles[p.variant].direct) p = heuristic_plan(g.npix, d->K, g.ntaps * d->cb, true, true, d->sh * d->sw > 1);
     p.splits = 1;
     if (d->cb == 4) return conv_c4_direct(kWhat, p, d, g, data, weight, bias, scale, false, out, s);
     return conv_s8_direct(kWhat, p, d, g, data, weight, bias, scale, out, s);
