@@ -81,7 +81,7 @@ extern "C" int unit_conv2d_nchw16c_f16f32(const unit_conv_desc *d, const void *a
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int ntable = (int)(sizeof(kTunedF16) / sizeof(kTunedF16[0])) - 1;
   // no k-splits: fp32 atomics would make the summation order, and so the result, vary run to run
-  const ConvPlan p = plan_conv(d, g.npix, g.ntaps * 32, kTunedF16, ntable, false, true);
+  const ConvPlan p = plan_conv(d, g.npix, g.ntaps * 32, kTunedF16, ntable, false, true, true);
   if (kConvTiles[p.variant].direct) return conv_f16_direct(p, d, g, a, b, out, s);
   return run_conv_f16_variant(p, d, g, a, b, out, s);
 }

@@ -44,7 +44,8 @@ struct TunedConv {
 // layers (few input channels, many pixels) want 64..128-pixel tiles of 64 channels with many
 // workgroups in flight; long reductions want the 128-channel tiles with two stages of loads in
 // flight; the 256 x 256 tiles only pay when they still give every CU several workgroups.
-inline ConvPlan heuristic_plan(int npix, int K, int kbytes, bool allow_split, bool direct_ok, bool strided = false) {
+inline ConvPlan heuristic_plan(int npix, int K, int kbytes, bool allow_split, bool direct_ok, bool strided = false,
+                               bool staged_too = false) {
   const bool k128 = kbytes % 128 == 0;
   const auto tiles = [&](int bx, int by) { return (long)ceil_div(K, bx) * ceil_div(npix, by); };
   if (direct_ok) {
@@ -75,6 +76,13 @@ inline ConvPlan heuristic_plan(int npix, int K, int kbytes, bool allow_split, bo
     } else {  // the fp16 operator (a k-step is one tap of 16 channels), same source
       const int nsteps = kbytes / 32;
       const bool wide = K % 128 == 0;
+      // Weights in the reference's layout (staged_too): with a reduction of 32 steps or more and enough large tiles
+      // the staged kernels, which share both operands through LDS, beat the direct ones (batch 256: 3 x 3 256 -> 256
+      // on 14 x 14 in 69 against 122 us; measured gain 5 - 45 % from 98 tiles of 256 x 256 up, a loss below)
+      if (staged_too && nsteps >= 32) {
+        if (K % 256 == 0 && tiles(256, 256) >= 196) return ConvPlan{0, 1, 0};
+        if (wide && tiles(256, 256) >= 98) return ConvPlan{18, 1, 0};
+      }
       if (t64 < 196)
         v = 60;
       else if (t64 < 392)
@@ -113,8 +121,8 @@ inline ConvPlan heuristic_plan(int npix, int K, int kbytes, bool allow_split, bo
 }
 
 inline ConvPlan plan_conv(const unit_conv_desc *d, int npix, int kbytes, const TunedConv *table, int ntable,
-                          bool allow_split, bool direct_ok) {
-  ConvPlan p = heuristic_plan(npix, d->K, kbytes, allow_split, direct_ok, d->sh * d->sw > 1);
+                          bool allow_split, bool direct_ok, bool staged_too = false) {
+  ConvPlan p = heuristic_plan(npix, d->K, kbytes, allow_split, direct_ok, d->sh * d->sw > 1, staged_too);
   // UNIT_AMD_CONV_NOTABLE=1: heuristic only (the tuner measures it as the baseline)
   if (tuning_override("UNIT_AMD_CONV_NOTABLE") > 0) ntable = 0;
   for (int i = 0; i < ntable; ++i) {
