@@ -188,6 +188,9 @@ int unit_prepack_conv_weight_f16(const void *src, void *dst, int32_t O, int32_t 
  * unit_gemm_f16_prepared: c (M, N) = a (M, K) . bt^T, same results as unit_gemm_f16 (the same
  * products summed in the same order); K % 8 == 0, N % 4 == 0. */
 int unit_gemm_f16_prepare_b(const void *b, void *bt, int32_t K, int32_t N, unit_stream_t stream);
+/* The same bt from a b that is already in the reference's packed form (apps/gpu/gemm-pack.py:9,17):
+ * bp f16 (N/32, K/32, 32, 32), bp[y/32][k/32][k%32][y%32] = b[k][y]; K % 32 == 0, N % 32 == 0. */
+int unit_gemm_f16_prepare_b_packed32(const void *bp, void *bt, int32_t K, int32_t N, unit_stream_t stream);
 int unit_gemm_f16_prepared(const void *a, const void *bt, void *c, int32_t M, int32_t N, int32_t K,
                            int32_t out_f16, unit_stream_t stream);
 

@@ -306,6 +306,27 @@ def gemm_f16(a, b):
     return a.astype(np.float64) @ b.astype(np.float64)
 
 
+def pack_gemm_b32(b):
+    """The packed operand of apps/gpu/gemm-pack.py:9,17: bp[y/32][k/32][k%32][y%32] = b[k][y], b (K, N)."""
+    k, n = b.shape
+    assert k % 32 == 0 and n % 32 == 0
+    return np.ascontiguousarray(b.reshape(k // 32, 32, n // 32, 32).transpose(2, 0, 1, 3))
+
+
+def gemm_f16_packed(a, bp):
+    """apps/gpu/gemm-pack.py:14-18: c[x,y] = sum_k f32(a[x,k]) * f32(bp[y/32, k/32, k%32, y%32]), in float64 on the
+    fp16-rounded inputs, as explicit index arithmetic (no reshape shared with pack_gemm_b32)."""
+    m, k = a.shape
+    nb, kb, k32, n32 = bp.shape
+    assert (k32, n32) == (32, 32) and kb * 32 == k
+    ks = np.arange(k)
+    out = np.empty((m, nb * 32), dtype=np.float64)
+    a64 = a.astype(np.float64)
+    for y in range(nb * 32):
+        out[:, y] = a64 @ bp[y // 32, ks // 32, ks % 32, y % 32].astype(np.float64)
+    return out
+
+
 def conv2d_nchw16c_f16(a, b, stride_h=1, stride_w=1):
     """python/tensorizer/ops/gpu.py:35-53: valid conv (no padding argument),
     O[n,ko,x,y,ob] = sum_{rc,rh,rw} a[n,rc/16,sh*x+rh,sw*y+rw,rc%16] * b[ko,rc/16,rh,rw,rc%16,ob],

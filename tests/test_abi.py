@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), f"libunit_amd.so does not export {n}"
     assert sorted(_lib.SYMBOLS) == names, "unit_amd/_lib.py and include/unit_amd.h disagree"
-    assert lib.unit_version() == 102
+    assert lib.unit_version() == 103
 
 
 def test_conv_desc_matches_the_header_struct():
@@ -119,6 +119,9 @@ def test_out_hw_and_error_paths_without_gpu():
     assert L.unit_gemm_f16(16, 2, 16, 16, 16, 16, 0, None) == -1 and b"aligned" in L.unit_last_error()
     # fp16 GEMM on a prepared b
     assert L.unit_gemm_f16_prepare_b(16, 16, 12, 16, None) == -1 and b"multiple of 8" in L.unit_last_error()
+    assert L.unit_gemm_f16_prepare_b_packed32(16, 16, 48, 64, None) == -1 and b"multiples of 32" in L.unit_last_error()
+    assert L.unit_gemm_f16_prepare_b_packed32(16, None, 64, 64, None) == -1 and b"null" in L.unit_last_error()
+    assert L.unit_gemm_f16_prepare_b_packed32(16, 8, 64, 64, None) == -1 and b"aligned" in L.unit_last_error()
     assert L.unit_gemm_f16_prepared(16, 16, 16, 16, 6, 16, 0, None) == -1 and b"multiple of 4" in L.unit_last_error()
     assert L.unit_gemm_f16_prepared(16, None, 16, 16, 8, 16, 0, None) == -1 and b"null" in L.unit_last_error()
     assert L.unit_gemm_f16_prepared(16, 8, 16, 16, 8, 16, 0, None) == -1 and b"aligned" in L.unit_last_error()

@@ -104,6 +104,27 @@ def test_gemm_fp16_prepared_b_integer_exact(dev, oracle):
         assert kernel in U.last_variant(), U.last_variant()  # registers; 256 x 128 hybrid; 256 x 256 all direct-to-LDS
 
 
+@pytest.mark.parametrize("M,N,K", [(64, 192, 1024), (128, 768, 3072), (300, 2080, 96), (4096, 4096, 512)])
+def test_gemm_fp16_reference_packed_b(dev, oracle, M, N, K):
+    """b handed over as the reference packs it, (N/32, K/32, 32, 32) (apps/gpu/gemm-pack.py:9,17; its own size is
+    64 x 192 x 1024): prepared once and passed straight to gemm_fp16, against the oracle's packed GEMM; with
+    integer-valued operands the result is exact and the re-laid operand equals b transposed."""
+    a = rng.normal_f16((M, K), 6100 + M)
+    b = rng.normal_f16((K, N), 6200 + N, 1.0 / np.sqrt(K))
+    bp = oracle.pack_gemm_b32(b)
+    tbp = _t(bp, dev)
+    prepared = U.prepare_gemm_b(tbp)
+    assert U.last_variant() == "f16_unpack32_b"
+    assert np.array_equal(prepared.bt.cpu().numpy(), b.T)
+    ref = oracle.gemm_f16_packed(a, bp) if M * N * K <= 1 << 28 else oracle.gemm_f16(a, b)
+    for out in (U.gemm_fp16(_t(a, dev), prepared), U.gemm_fp16(_t(a, dev), tbp)):
+        assert max_rel(out.cpu().numpy(), ref) <= REL_TOL, U.last_variant()
+    ai = (np.arange(M * K).reshape(M, K) % 7).astype(np.float16)
+    bi = (np.arange(K * N).reshape(K, N) % 5 - 2).astype(np.float16)
+    out = U.gemm_fp16(_t(ai, dev), _t(oracle.pack_gemm_b32(bi), dev)).cpu().numpy()
+    assert np.array_equal(out.astype(np.float64), oracle.gemm_f16(ai, bi)), U.last_variant()
+
+
 def test_gemm_fp16_integer_exact(dev, oracle):
     """Small-integer operands (the arange % 7 recipe of apps/gpu/conv-wdim.py:33-36) make every
     fp32 partial sum exact, so the result must match the float64 reference bit for bit."""

@@ -298,6 +298,20 @@ def test_fp16_golden_and_integer_exact(oracle):
     assert np.array_equal(oracle.gemm_f16(a, b), (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float64))
 
 
+def test_fp16_gemm_packed_b(oracle):
+    """The packed operand of apps/gpu/gemm-pack.py:9,17 against its defining index formula, element by element,
+    and the packed GEMM against the plain one on the same b (integer-valued operands: exact)."""
+    k, n = 64, 96
+    b = (np.arange(k * n).reshape(k, n) % 11 - 5).astype(np.float16)
+    bp = oracle.pack_gemm_b32(b)
+    assert bp.shape == (n // 32, k // 32, 32, 32)
+    for y in range(n):
+        for kk in range(k):
+            assert bp[y // 32, kk // 32, kk % 32, y % 32] == b[kk, y]
+    a = (np.arange(5 * k).reshape(5, k) % 7).astype(np.float16)
+    assert np.array_equal(oracle.gemm_f16_packed(a, bp), oracle.gemm_f16(a, b))
+
+
 def test_fp16_conv_matches_torch_double(oracle):
     g = np.load(os.path.join(GOLD, "fp16_conv_3x3_c32_k32.npz"))
     assert np.array_equal(oracle.conv2d_nchw16c_f16(g["a"], g["b"], 1, 1), g["out"])

@@ -24,6 +24,7 @@ SYMBOLS = (
     "unit_dense_u8s8s32",
     "unit_gemm_f16",
     "unit_gemm_f16_prepare_b",
+    "unit_gemm_f16_prepare_b_packed32",
     "unit_gemm_f16_prepared",
     "unit_conv2d_nchw16c_f16f32",
     "unit_pack_nchwc",
@@ -86,6 +87,7 @@ def load():
     L.unit_dense_u8s8s32.argtypes = [vp, vp, vp, i32, i32, i32, vp]
     L.unit_gemm_f16.argtypes = [vp, vp, vp, i32, i32, i32, i32, vp]
     L.unit_gemm_f16_prepare_b.argtypes = [vp, vp, i32, i32, vp]
+    L.unit_gemm_f16_prepare_b_packed32.argtypes = [vp, vp, i32, i32, vp]
     L.unit_gemm_f16_prepared.argtypes = [vp, vp, vp, i32, i32, i32, i32, vp]
     L.unit_conv2d_nchw16c_f16f32.argtypes = [dp, vp, vp, vp, vp]
     L.unit_pack_nchwc.argtypes = [vp, vp, i32, i32, i32, i32, i32, i32, vp]

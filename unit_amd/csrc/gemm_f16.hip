@@ -128,6 +128,18 @@ __global__ __launch_bounds__(256) void transpose_f16(const _Float16 *__restrict_
     if (n0 + r < N && k0 + tx < K) bt[(size_t)(n0 + r) * K + k0 + tx] = tile[tx][r];
 }
 
+// bp (N/32, K/32, 32, 32) with bp[y/32][k/32][k%32][y%32] = b[k][y] (apps/gpu/gemm-pack.py:9,17) -> bt (N, K):
+// one 32 x 32 block (2 KiB, contiguous in bp) per workgroup, transposed through LDS; 64-byte row segments of bt
+__global__ __launch_bounds__(256) void unpack32_f16(const _Float16 *__restrict__ bp, _Float16 *__restrict__ bt, int K) {
+  __shared__ _Float16 tile[32][34];
+  const int kb = blockIdx.x, nb = blockIdx.y;
+  const _Float16 *src = bp + ((size_t)nb * gridDim.x + kb) * 1024;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  for (int r = ty; r < 32; r += 8) tile[r][tx] = src[r * 32 + tx];  // tile[k % 32][y % 32]
+  __syncthreads();
+  for (int r = ty; r < 32; r += 8) bt[(size_t)(nb * 32 + r) * K + kb * 32 + tx] = tile[tx][r];
+}
+
 // TAIL = false: K is a whole number of stages (the loaders then stage without zeroing selects)
 template <class T, bool OUT_F16, int PF = 1, bool TAIL = true>
 int run_gemm_f16(const void *a, const void *b, void *c, int M, int N, int K, hipStream_t s) {
@@ -222,6 +234,24 @@ extern "C" int unit_gemm_f16_prepare_b(const void *b, void *bt, int32_t K, int32
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "%s: launch: %s", what, hipGetErrorString(e));
   set_variant("f16_transpose_b");
+  return UNIT_OK;
+}
+
+extern "C" int unit_gemm_f16_prepare_b_packed32(const void *bp, void *bt, int32_t K, int32_t N, unit_stream_t stream) {
+  using namespace unit;
+  const char *what = "unit_gemm_f16_prepare_b_packed32";
+  if (!bp || !bt) return fail(UNIT_E_ARG, "%s: null pointer", what);
+  if (K <= 0 || N <= 0) return fail(UNIT_E_ARG, "%s: K, N must be positive (got %d, %d)", what, K, N);
+  if (K % 32 || N % 32) return fail(UNIT_E_ARG, "%s: K and N must be multiples of 32 (got %d, %d)", what, K, N);
+  if (!fits((size_t)N * K * 2)) return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
+  if (N / 32 > 65535) return fail(UNIT_E_ARG, "%s: N exceeds 32 * 65535", what);
+  if (int rc = check_aligned(what, {bp, bt})) return rc;
+  if (int rc = check_device()) return rc;
+  hipLaunchKernelGGL(unpack32_f16, dim3(K / 32, N / 32), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const _Float16 *>(bp), static_cast<_Float16 *>(bt), K);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "%s: launch: %s", what, hipGetErrorString(e));
+  set_variant("f16_unpack32_b");
   return UNIT_OK;
 }
 

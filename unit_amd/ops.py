@@ -385,8 +385,17 @@ class PreparedGemmB:
 
 def prepare_gemm_b(b):
     """Re-lay the constant operand b (K, N) of gemm_fp16 once as (N, K), the counterpart of the one-time
-    packing of b in apps/gpu/gemm-pack.py:9,17; gemm_fp16 accepts the result in place of b."""
-    b = _dev(b, "b", torch.float16, 2)
+    packing of b in apps/gpu/gemm-pack.py:9,17; gemm_fp16 accepts the result in place of b.  A 4-D b is taken
+    as that file's packed operand (N/32, K/32, 32, 32)."""
+    b = _dev(b, "b", torch.float16, (2, 4))
+    if b.dim() == 4:  # already packed as the reference packs it: (N/32, K/32, 32, 32), [y/32][k/32][k%32][y%32]
+        nb, kb, k32, n32 = b.shape
+        if (k32, n32) != (32, 32):
+            raise ValueError(f"b: a packed operand is (N/32, K/32, 32, 32), got {tuple(b.shape)}")
+        k, n = kb * 32, nb * 32
+        bt = torch.empty((n, k), dtype=torch.float16, device=b.device)
+        check(_lib.load().unit_gemm_f16_prepare_b_packed32(b.data_ptr(), bt.data_ptr(), k, n, _stream()))
+        return PreparedGemmB(bt, k, n)
     k, n = b.shape
     bt = torch.empty((n, k), dtype=torch.float16, device=b.device)
     check(_lib.load().unit_gemm_f16_prepare_b(b.data_ptr(), bt.data_ptr(), k, n, _stream()))
@@ -395,12 +404,15 @@ def prepare_gemm_b(b):
 
 def gemm_fp16(a, b, out_dtype="float32"):
     """c[x, y] = sum_k f32(a[x, k]) * f32(b[k, y]); a (M, K), b (K, N) fp16 row-major, or b a
-    PreparedGemmB."""
+    PreparedGemmB, or b packed (N/32, K/32, 32, 32) with b4[y/32][k/32][k%32][y%32] = b[k][y] as
+    apps/gpu/gemm-pack.py:9,14-18 takes it (re-laid on every call: prepare it once instead)."""
     a = _dev(a, "a", torch.float16, 2)
     if out_dtype not in ("float32", "float16"):
         raise ValueError(f"out_dtype: expected 'float32' or 'float16', got {out_dtype!r}")
     m, k = a.shape
     half = out_dtype == "float16"
+    if isinstance(b, torch.Tensor) and b.dim() == 4:
+        b = prepare_gemm_b(b)
     if isinstance(b, PreparedGemmB):
         if b.K != k or b.bt.device != a.device:
             raise ValueError(f"b: {b!r} does not match a {tuple(a.shape)} on {a.device}")
