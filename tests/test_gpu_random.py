@@ -1,7 +1,7 @@
 """Random shapes through every entry point against the oracle: convolutions (16- and 4-channel blocks, strides,
 asymmetric padding, dilation, ragged sizes; reference layout, prepared weights, the fused form, its NCHW store, the
-requantised form, the fp16 operator), the int8 dense and the fp16 GEMM (both layouts of the constant operand, both
-output types) and the layout kernels.  Every fourth case runs with the tuned tables switched off.  int8 is compared
+requantised form, the fp16 operator), conv3d, the int8 dense and the fp16 GEMM (every layout of the constant operand,
+both output types) and the layout kernels.  Every fourth case runs with the tuned tables switched off.  int8 is compared
 bit for bit, fp16 within the stated tolerance.  A failure names its case by (block, index, shape, seed)."""
 import numpy as np
 import pytest
@@ -118,6 +118,30 @@ def _run_gemm(O, dev, cs, seed):
         assert _rel(out.float().cpu().numpy(), ref16) <= REL_TOL, ("gemm", out_dtype, U.last_variant())
         out = U.gemm_fp16(ta, U.prepare_gemm_b(tb), out_dtype)
         assert _rel(out.float().cpu().numpy(), ref16) <= REL_TOL, ("gemm, prepared b", out_dtype, U.last_variant())
+    if n % 32 == 0 and k % 32 == 0:  # b as the reference packs it, (N/32, K/32, 32, 32)
+        out = U.gemm_fp16(ta, t(O.pack_gemm_b32(b16)))
+        assert _rel(out.cpu().numpy(), ref16) <= REL_TOL, ("gemm, packed b", U.last_variant())
+
+
+def _conv3d_case(r):
+    cb = 16 if r.rand() < 0.75 else 4
+    c = 16 * int(r.randint(1, 9)) if cb == 16 else 4 * int(r.choice([1, 2, 3]))
+    n = int(r.choice([1, 2, 3]))
+    d, h, w = int(r.randint(1, 9)), int(r.randint(1, 15)), int(r.randint(1, 15))
+    k = 16 * int(r.randint(1, 9))
+    kd, kh, kw = int(r.randint(1, 4)), int(r.randint(1, 4)), int(r.randint(1, 4))
+    if kd > d or kh > h or kw > w or (cb == 16 and kd * kh * kw > 31):
+        return None
+    return dict(cb=cb, c=c, n=n, d=d, h=h, w=w, k=k, kd=kd, kh=kh, kw=kw, stride=int(r.randint(1, 3)))
+
+
+def _run_conv3d(O, dev, cs, seed):
+    g = np.random.RandomState(seed)
+    cb = cs["cb"]
+    data = g.randint(-128, 128, (cs["n"], cs["c"] // cb, cs["d"], cs["h"], cs["w"], cb)).astype(np.int8)
+    wt = g.randint(-128, 128, (cs["k"] // 16, cs["c"] // cb, cs["kd"], cs["kh"], cs["kw"], cb // 4, 16, 4)).astype(np.int8)
+    out = U.conv3d_NCDHWc_int8(torch.from_numpy(data).to(dev), torch.from_numpy(wt).to(dev), cs["stride"])
+    assert np.array_equal(out.cpu().numpy(), O.conv3d_ncdhwc_int8(data, wt, cs["stride"])), ("conv3d", U.last_variant())
 
 
 def _layout_case(r):
@@ -136,11 +160,11 @@ def _run_layout(O, dev, cs, seed):
 @pytest.mark.parametrize("block", range(8))
 def test_random_cases(dev, oracle, block, monkeypatch):
     r = np.random.RandomState(52000 + block)
-    make = {"conv": _conv_case, "gemm": _gemm_case, "layout": _layout_case}
-    run = {"conv": _run_conv, "gemm": _run_gemm, "layout": _run_layout}
+    make = {"conv": _conv_case, "gemm": _gemm_case, "layout": _layout_case, "conv3d": _conv3d_case}
+    run = {"conv": _run_conv, "gemm": _run_gemm, "layout": _run_layout, "conv3d": _run_conv3d}
     done = 0
     while done < CASES_PER_BLOCK:
-        kind = str(r.choice(["conv", "conv", "conv", "conv", "gemm", "layout"]))
+        kind = str(r.choice(["conv", "conv", "conv", "conv", "gemm", "layout", "conv3d"]))
         cs = make[kind](r)
         if cs is None:
             continue
