@@ -121,12 +121,13 @@ def prepack_conv_weight(w, cb):
     return np.ascontiguousarray(t.transpose(0, 2, 5, 6, 3, 1, 4))
 
 
-def prepack_dense_weight(w):
-    """(N, K) -> (N/128, K/4, 128, 4), Wp[n/128, k/4, n%128, k%4] = W[n, k]
-    (shape from apps/cpu/kernel/int8-gemm.py:14; 16x4 analogue poc/vnni/vnni_dense.py:10-11)."""
+def prepack_dense_weight(w, tile=128):
+    """(N, K) -> (N/tile, K/4, tile, 4), Wp[n/tile, k/4, n%tile, k%4] = W[n, k]
+    (tile 128: shape from apps/cpu/kernel/int8-gemm.py:14; tile 16: the reference's own statement of the order,
+    poc/vnni/vnni_dense.py:10-11 `packed[w, x, y, z] = b[w * 16 + y, x * 4 + z]`)."""
     n, k = w.shape
-    assert n % 128 == 0 and k % 4 == 0
-    return np.ascontiguousarray(w.reshape(n // 128, 128, k // 4, 4).transpose(0, 2, 1, 3))
+    assert n % tile == 0 and k % 4 == 0
+    return np.ascontiguousarray(w.reshape(n // tile, tile, k // 4, 4).transpose(0, 2, 1, 3))
 
 
 def prepack_conv_weight_f16(w):

@@ -137,3 +137,74 @@ def test_tuned_tables_name_existing_variants():
             keys.add((npix, k, c, kh, kw, sh))
             if path.endswith("_prepared.inc"):
                 assert L.unit_conv_variant_is_direct(variant) == 1, (path, row)
+
+
+def test_registry_keeps_the_reference_fragment_keys():
+    # python/tensorizer/intrinsics/intrinsics.py:28-39
+    for key in ("tensorcore.load_a", "tensorcore.load_b", "tensorcore.store_c"):
+        assert U.INTRINSICS[key]["part_of"] is U.INTRINSICS["mfma.f16"]
+
+
+def test_bench_final_line_fits_the_tail_budget():
+    """The driver keeps a tail of a few KiB of stdout: the last line must be one complete JSON object under 2 KiB
+    even with every field at a plausible maximum width."""
+    import json
+
+    import bench
+    line = {
+        "metric": "int8 conv2d TOPS & % int8 MFMA peak (ResNet-50 b32); fp16 GEMM TFLOPS", "value": 123456.78,
+        "unit": "TOP/s", "n_gpus": 1, "steps": 1000, "warmup": 100, "ms_per_step": 1234.5678, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": "ResNet-50 v1 conv stack (53 convs, 20 shapes), batch 32, int8 u8 x s8 -> i32, "
+                               "NCHW16c / NCHW4c stem (BASELINE.json configs[4])",
+                   "batch": 32, "ops_per_step": 246779215872, "weights": "prepared"},
+        "pct_int8_mfma_peak": 99.99, "bit_exact_vs_oracle": True,
+        "roofline": dict(bound="hbm", achieved=4412.8, peak=8000.0, unit="GB/s", frac=0.5516, frac_cold=0.5012,
+                         traffic=115840483, traffic_source="profiles/conv_i8_resnet50_b32_1x1_64_256_56.txt",
+                         kernel="i8prep_c16_x64_y64_g1_d2w4n_r2_s1", layer="1x1s2_1024_2048@14", launch_us=24.75,
+                         launch_us_cold=26.11),
+        "cpu_baseline": dict(value=5.634, unit="TOP/s", cores=16, kind="port", vnni=True,
+                             sample="same step by the AVX-512 VNNI oracle: 20 unique layers, warm-up + repeat=10 x "
+                                    "number=3 each, mean x multiplicity",
+                             seconds=0.044, gemm_int8_tops=17.61, gemm_fp16_tflops=1.31),
+        "best_mfma_bound_layer": dict(layer="3x3_512_512@7", us=9.67, pct_int8_peak=15.2),
+        "gemm_int8_us": 80.39, "gemm_int8_pct_peak": 33.97, "gemm_fp16_us": 143.58, "gemm_fp16_tflops": 957.2,
+        "gemm_fp16_pct_peak": 38.05, "gemm_fp16_prepared_b_us": 119.64, "gemm_fp16_prepared_b_pct_peak": 45.66,
+        "gemm_fp16_max_rel_err": 0.000247, "sum_layers_cold_us": 612.3, "launch": "hipgraph",
+        "fp16_conv": dict(stack_us=618.2, tflops=387.0),
+        "probe": {"int8_tops": 4409.7, "fp16_tflops": 2327.2, "int8_tops_random_operands": 3374.3,
+                  "fp16_tflops_random_operands": 1646.7},
+    }
+    s = bench.compact_line(dict(line))
+    assert len(s) <= bench.FINAL_LINE_BUDGET and "\n" not in s
+    back = json.loads(s)
+    for key in ("metric", "value", "unit", "ms_per_step", "roofline", "cpu_baseline", "config"):
+        assert key in back
+    # an oversized line sheds optional keys, never the contract's
+    line["probe"] = {f"k{i}": "x" * 40 for i in range(40)}
+    back = json.loads(bench.compact_line(dict(line)))
+    assert "probe" not in back and "roofline" in back and "cpu_baseline" in back
+
+
+def test_bench_traffic_table_names_its_profiles():
+    import os
+
+    import bench
+    table = bench.read_traffic_table()
+    assert table, "profiles/hbm_traffic_table.txt is missing or empty"
+    for (layer, kernel), (nbytes, src) in table.items():
+        assert any(s.name == layer for s in WL.RESNET50) and nbytes > 0
+        assert os.path.exists(os.path.join(os.path.dirname(bench.__file__), src)), src
+
+
+def test_padding_bound_is_checked_on_the_host():
+    import ctypes
+
+    from unit_amd import _lib
+    L = _lib.load()
+    oh, ow = ctypes.c_int32(), ctypes.c_int32()
+    ok = _lib.ConvDesc(1, 16, 8, 8, 16, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 16)
+    assert L.unit_conv_out_hw(ctypes.byref(ok), ctypes.byref(oh), ctypes.byref(ow)) == 0 and (oh.value, ow.value) == (8, 8)
+    bad = _lib.ConvDesc(1, 16, 8, 8, 16, 3, 3, 1, 1, 16384, 1, 1, 1, 1, 1, 16)
+    assert L.unit_conv_out_hw(ctypes.byref(bad), ctypes.byref(oh), ctypes.byref(ow)) != 0
+    assert b"padding" in L.unit_last_error()

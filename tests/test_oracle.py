@@ -343,3 +343,31 @@ def test_requant_definition_small_cases(oracle):
     ident = oracle.conv2d_nchwc_u8_requant(x, w, bias, 1 << 8, 16, 1, 1, 1)   # (acc * 256 + 2**15) >> 16 = round(acc / 256)
     assert np.array_equal(ident, np.clip(np.floor(acc / 256.0 + 0.5), 0, 255).astype(np.uint8))
     assert (oracle.conv2d_nchwc_u8_requant(x, w, bias, 5, 3, 1, 1, 1)[acc < -1] == 0).all()
+
+
+def test_dense_pack_order_is_the_reference_lambda_at_tile_16(oracle):
+    """poc/vnni/vnni_dense.py:10-11 states the packed order literally, for 16-row tiles:
+    packed[w, x, y, z] = b[w * 16 + y, x * 4 + z]; and :17-19 the product through it:
+    c[x, y] = sum_k packed_a[x // 16, k // 4, x % 16, k % 4] * packed_b[y // 16, k // 4, y % 16, k % 4].
+    The oracle's pack at tile 16 must be that lambda, element by element; tile 128 is the same rule."""
+    from unit_amd import rng
+    n, k = 48, 24
+    b = rng.uniform_s8((n, k), 77)
+    got = oracle.prepack_dense_weight(b, tile=16)
+    assert got.shape == (n // 16, k // 4, 16, 4)
+    for w in range(n // 16):
+        for x in range(k // 4):
+            for y in range(16):
+                for z in range(4):
+                    assert got[w, x, y, z] == b[w * 16 + y, x * 4 + z]
+    a = rng.uniform_s8((32, k), 78)
+    pa = oracle.prepack_dense_weight(a, tile=16)
+    c = np.zeros((32, n), np.int64)
+    for x in range(32):
+        for y in range(n):
+            c[x, y] = sum(int(pa[x // 16, r // 4, x % 16, r % 4]) * int(got[y // 16, r // 4, y % 16, r % 4]) for r in range(k))
+    assert np.array_equal(c, a.astype(np.int64) @ b.astype(np.int64).T)
+    # the 128-row form follows the same rule
+    b2 = rng.uniform_s8((256, 8), 79)
+    g2 = oracle.prepack_dense_weight(b2)
+    assert all(g2[w, x, y, z] == b2[w * 128 + y, x * 4 + z] for w in range(2) for x in range(2) for y in (0, 5, 127) for z in range(4))

@@ -43,6 +43,10 @@ static int out_hw(const unit_conv_desc *d, int *OH, int *OW, const char *what) {
   if (d->sh <= 0 || d->sw <= 0 || d->dh <= 0 || d->dw <= 0)
     return fail(UNIT_E_ARG, "%s: strides and dilations must be positive", what);
   if (d->pt < 0 || d->pl < 0 || d->pb < 0 || d->pr < 0) return fail(UNIT_E_ARG, "%s: negative padding", what);
+  // the staged loaders mark a tap past the reduction end by a row offset of 32767, which must stay outside the
+  // padded image for every output row
+  if (d->pt >= 16384 || d->pl >= 16384 || d->pb >= 16384 || d->pr >= 16384)
+    return fail(UNIT_E_ARG, "%s: padding of 16384 or more is not supported", what);
   const long eh = (long)d->H + d->pt + d->pb - (long)d->dh * (d->KH - 1) - 1;
   const long ew = (long)d->W + d->pl + d->pr - (long)d->dw * (d->KW - 1) - 1;
   if (eh < 0 || ew < 0) return fail(UNIT_E_ARG, "%s: kernel window larger than the padded input", what);

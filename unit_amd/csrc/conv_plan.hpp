@@ -127,10 +127,20 @@ inline ConvPlan plan_conv(const unit_conv_desc *d, int npix, int kbytes, const T
   if (tuning_override("UNIT_AMD_CONV_NOTABLE") > 0) ntable = 0;
   for (int i = 0; i < ntable; ++i) {
     const TunedConv &e = table[i];
-    if (e.npix == npix && e.K == d->K && e.C == d->C && e.KH == d->KH && e.KW == d->KW && e.sh == d->sh) {
+    // the tables were tuned on square strides without dilation; a direct choice needs a window the direct
+    // kernels can run, otherwise the heuristic's (staged) choice stands
+    if (e.npix == npix && e.K == d->K && e.C == d->C && e.KH == d->KH && e.KW == d->KW && e.sh == d->sh &&
+        d->sw == d->sh && d->dh == 1 && d->dw == 1 && (direct_ok || !kConvTiles[e.variant].direct)) {
       p = ConvPlan{e.variant, e.splits, e.panel};
       break;
     }
+  }
+  // A direct variant whose k-groups park one float tile each can outgrow the LDS on very deep reductions (the tap
+  // table follows the tiles): the one-wave six-deep kernel of the same family always fits.
+  if (!allow_split && kConvTiles[p.variant].direct && kConvTiles[p.variant].kg > 1) {
+    const TileShape &t = kConvTiles[p.variant];
+    const long tile = (long)t.bx * t.by * 4 + t.bx * 4, scratch = 32 * 144 + 128;  // DirectShape: TILE + WSUM, kScratch
+    if (t.kg * (scratch + tile) + (long)(kbytes / 32) * 8 > kMaxLds) p = ConvPlan{68, 1, p.panel};
   }
   const int ov = tuning_override("UNIT_AMD_CONV_VARIANT"), os = tuning_override("UNIT_AMD_CONV_SPLITK");
   if (ov > 0 && ov <= kNumConvTiles) p.variant = ov - 1;

@@ -32,3 +32,16 @@ INTRINSICS = {
 # the reference's own keys resolve to the back end that took their place
 INTRINSICS["vnni"] = INTRINSICS["mfma.i8"]
 INTRINSICS["tensorcore"] = INTRINSICS["mfma.f16"]
+# The reference registers the wmma fragment moves as intrinsics of their own ('tensorcore.load_a', '.load_b',
+# '.store_c': intrinsics.py:28-39, emitters intrinsics/gpu.py:104-113,197-216).  Here they are steps inside the
+# kernels, not callable operators; the keys stay so that a lookup by the reference's names says what took their place.
+INTRINSICS["tensorcore.load_a"] = {
+    "pattern": {"instruction": "global_load_lds_dwordx4 + ds_read_b128", "tile": (32, 16), "dtype": "float16"},
+    "replaces": "llvm.nvvm.wmma.m16n16k16.load.a.row.stride.f16", "part_of": INTRINSICS["mfma.f16"]}
+INTRINSICS["tensorcore.load_b"] = {
+    "pattern": {"instruction": "global_load_lds_dwordx4 + ds_read_b128", "tile": (32, 16), "dtype": "float16"},
+    "replaces": "llvm.nvvm.wmma.m16n16k16.load.b.row.stride.f16", "part_of": INTRINSICS["mfma.f16"]}
+INTRINSICS["tensorcore.store_c"] = {
+    "pattern": {"instruction": "global_store_dwordx4 (non-temporal) from the accumulators", "tile": (32, 32),
+                "dtype": "float32"},
+    "replaces": "llvm.nvvm.wmma.m16n16k16.store.d.row.stride.f32", "part_of": INTRINSICS["mfma.f16"]}
