@@ -10,9 +10,11 @@ tree).  What pins each function is listed in the header of tests/test_oracle.py.
 Parity status:
   * conv2d / stencil / layouts / pre-pack / fp16: pinned (known-answer vector, brute force,
     independent library routine, printed transform chain).
-  * dense packed-weight *index order*: PARITY UNPINNED -- the reference gives only the
-    placeholder shape (N/128, K/4, 128, 4) (apps/cpu/kernel/int8-gemm.py:14) and never
-    checks values through it.  The logical product a . W^T is pinned.
+  * dense packed-weight *index order*: pinned at tile 16 by the reference's own literal index
+    lambda (poc/vnni/vnni_dense.py:10-11, checked element by element); for the 128-row tile the
+    reference gives only the placeholder shape (N/128, K/4, 128, 4) (apps/cpu/kernel/
+    int8-gemm.py:14), read here as the same rule with 128 in place of 16 -- that reading stays
+    PARITY UNPINNED.  The logical product a . W^T is pinned.
   * fused signed form with spatial padding: PARITY UNPINNED (the reference's printed graphs have
     padding 0; zero padding of the signed data follows upstream TVM).
   * conv2d_nchwc_u8_requant: PARITY UNPINNED -- an extension with no counterpart in the

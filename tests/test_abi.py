@@ -80,15 +80,16 @@ def test_out_hw_and_error_paths_without_gpu():
     assert L.unit_conv3d_ncdhwc_s8s8s32(ctypes.byref(d3), 1, 1, 1, None) == -1 and b"window" in L.unit_last_error()
     assert L.unit_conv_variant_count() >= 70
     kinds = [L.unit_conv_variant_is_direct(v) for v in range(L.unit_conv_variant_count())]
-    assert set(kinds) == {0, 1} and kinds.count(1) >= 20
+    assert set(kinds) == {0, 1, 2} and kinds.count(1) >= 20 and kinds.count(2) >= 4
     assert L.unit_conv_variant_is_direct(-1) == -1 and L.unit_conv_variant_is_direct(len(kinds)) == -1
-    # prepared weights: size formula ceil(K/32) * k-steps * 1 KiB (+ 128 bytes of addends per block for int8)
+    # prepared weights: size formula ceil(K/32) * k-steps * 1 KiB (+ 128 bytes of addends per block and 16 KiB of
+    # zeros, the lines the LDS-shared kernels fetch for padded taps, for int8)
     nb = ctypes.c_size_t()
-    assert L.unit_conv2d_prepared_weight_bytes(256, 256, 3, 3, 16, 1, ctypes.byref(nb)) == 0 and nb.value == 8 * 72 * 1024 + 8 * 128
-    assert L.unit_conv2d_prepared_weight_bytes(48, 16, 3, 3, 16, 1, ctypes.byref(nb)) == 0 and nb.value == 2 * 5 * 1024 + 2 * 128
+    assert L.unit_conv2d_prepared_weight_bytes(256, 256, 3, 3, 16, 1, ctypes.byref(nb)) == 0 and nb.value == 8 * 72 * 1024 + 8 * 128 + 16384
+    assert L.unit_conv2d_prepared_weight_bytes(48, 16, 3, 3, 16, 1, ctypes.byref(nb)) == 0 and nb.value == 2 * 5 * 1024 + 2 * 128 + 16384
     assert L.unit_conv2d_prepared_weight_bytes(48, 16, 3, 3, 16, 2, ctypes.byref(nb)) == 0 and nb.value == 2 * 9 * 1024
     # 4-channel blocks: one k-step per (channel block, kh)
-    assert L.unit_conv2d_prepared_weight_bytes(64, 4, 7, 7, 4, 1, ctypes.byref(nb)) == 0 and nb.value == 2 * 7 * 1024 + 2 * 128
+    assert L.unit_conv2d_prepared_weight_bytes(64, 4, 7, 7, 4, 1, ctypes.byref(nb)) == 0 and nb.value == 2 * 7 * 1024 + 2 * 128 + 16384
     assert L.unit_conv2d_prepared_weight_bytes(64, 4, 9, 9, 4, 1, ctypes.byref(nb)) == -1 and b"KW <= 8" in L.unit_last_error()
     assert L.unit_conv2d_prepared_weight_bytes(64, 4, 3, 3, 4, 2, ctypes.byref(nb)) == -1 and b"cb must be" in L.unit_last_error()
     assert L.unit_conv2d_prepared_weight_bytes(40, 16, 3, 3, 16, 1, ctypes.byref(nb)) == -1 and b"multiple of 16" in L.unit_last_error()

@@ -172,6 +172,8 @@ def test_conv2d_every_variant(dev, oracle, monkeypatch, N, C, H, W, K, ks, strid
     assert count >= 40
     ran = set()
     for v in range(1, count + 1):
+        if _lib.load().unit_conv_variant_is_direct(v - 1) == 2:
+            continue  # LDS-shared variants exist for prepared weights only: the id runs the heuristic's choice here
         for splits in (1, 3):
             monkeypatch.setenv("UNIT_AMD_CONV_VARIANT", str(v))
             monkeypatch.setenv("UNIT_AMD_CONV_SPLITK", str(splits))

@@ -11,6 +11,7 @@ from unit_amd import rng
 pytestmark = pytest.mark.gpu
 
 REL_TOL = 1e-2
+ZERO_BYTES = 16384  # zero region behind prepared int8 weights
 
 
 def _t(a, dev):
@@ -53,9 +54,11 @@ def test_prepared_buffer_int8(dev, K, C, ks):
     torch.cuda.synchronize()
     frag, addend = _fragments_i8(wt)
     buf = p.buf.cpu().numpy()
-    assert buf.size == frag.size + addend.size * 4
+    # fragments, the 128 * sum(w) addends, then 16 KiB of zeros (what the LDS-shared kernels fetch for padded taps)
+    assert buf.size == frag.size + addend.size * 4 + ZERO_BYTES
     assert np.array_equal(buf[:frag.size].view(np.int8).reshape(frag.shape), frag)
-    assert np.array_equal(buf[frag.size:].view(np.int32), addend)
+    assert np.array_equal(buf[frag.size:buf.size - ZERO_BYTES].view(np.int32), addend)
+    assert not buf[buf.size - ZERO_BYTES:].any()
 
 
 @pytest.mark.parametrize("K,C,kh,kw", [(64, 4, 7, 7), (48, 8, 3, 3), (16, 4, 2, 8), (32, 12, 1, 5)])
@@ -74,9 +77,11 @@ def test_prepared_buffer_int8_c4(dev, K, C, kh, kw):
     addend = np.zeros(kblocks * 32, np.int32)
     addend[:K] = 128 * w.astype(np.int64).sum(axis=(1, 2, 3))
     buf = p.buf.cpu().numpy()
-    assert buf.size == frag.size + addend.size * 4
+    # fragments, the 128 * sum(w) addends, then 16 KiB of zeros (what the LDS-shared kernels fetch for padded taps)
+    assert buf.size == frag.size + addend.size * 4 + ZERO_BYTES
     assert np.array_equal(buf[:frag.size].view(np.int8).reshape(frag.shape), frag)
-    assert np.array_equal(buf[frag.size:].view(np.int32), addend)
+    assert np.array_equal(buf[frag.size:buf.size - ZERO_BYTES].view(np.int32), addend)
+    assert not buf[buf.size - ZERO_BYTES:].any()
 
 
 @pytest.mark.parametrize("K,C,ks", [(64, 64, 3), (48, 16, 1), (16, 48, 2)])
@@ -186,7 +191,8 @@ def test_conv2d_prepared_c4_every_direct_variant(dev, oracle, monkeypatch):
     (1, 48, 8, 8, 32, 3, 1, 0),     # 27 taps without padding
 ])
 def test_conv2d_prepared_every_direct_variant(dev, oracle, monkeypatch, N, C, H, W, K, ks, stride, pad):
-    """u8 and fused signed form on every direct variant (ids of staged variants fall back to a direct one)."""
+    """u8 and fused signed form on every direct and every LDS-shared variant (ids of register-staged variants fall
+    back to a direct one)."""
     from unit_amd import _lib
     data = rng.uniform_u8((N, C // 16, H, W, 16), 11 * C + H)
     xs = (data ^ 0x80).view(np.int8)
@@ -207,7 +213,8 @@ def test_conv2d_prepared_every_direct_variant(dev, oracle, monkeypatch, N, C, H,
         torch.cuda.synchronize()
         names.add(U.last_variant())
         assert np.array_equal(out.cpu().numpy(), ref_fused), (v, U.last_variant())
-    assert len(names) >= 30 and all(n.startswith(("i8prep", "s8prep")) for n in names), names
+    assert len(names) >= 30 and all(n.startswith(("i8prep", "s8prep", "i8lds", "s8lds")) for n in names), names
+    assert sum(n.startswith("i8lds") for n in names) >= 4 and sum(n.startswith("s8lds") for n in names) >= 4, names
 
 
 FP16_CASES = [
@@ -343,7 +350,7 @@ def test_conv2d_requant_every_direct_variant(dev, oracle, monkeypatch):
         torch.cuda.synchronize()
         names.add(U.last_variant())
         assert np.array_equal(out.cpu().numpy(), ref), (v, U.last_variant())
-    assert len(names) >= 15
+    assert len(names) >= 15 and sum(n.startswith("q8lds") for n in names) >= 4, names
 
 
 def test_conv_chain_through_requantised_activations(dev, oracle):

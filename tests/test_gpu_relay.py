@@ -98,7 +98,7 @@ def test_planar_store_on_every_direct_variant(dev):
     ran = 0
     try:
         for v in range(L.unit_conv_variant_count()):
-            if L.unit_conv_variant_is_direct(v) != 1:
+            if L.unit_conv_variant_is_direct(v) not in (1, 2):  # direct and LDS-shared variants take prepared weights
                 continue
             os.environ["UNIT_AMD_CONV_VARIANT"] = str(v + 1)
             try:

@@ -33,7 +33,7 @@ extern "C" int unit_conv_variant_count(void) { return unit::kNumConvTiles; }
 
 extern "C" int unit_conv_variant_is_direct(int32_t variant) {
   if (variant < 0 || variant >= unit::kNumConvTiles) return -1;
-  return unit::kConvTiles[variant].direct ? 1 : 0;
+  return unit::kConvTiles[variant].lds ? 2 : (unit::kConvTiles[variant].direct ? 1 : 0);
 }
 
 extern "C" int unit_conv2d_nchwc_u8s8s32(const unit_conv_desc *d, const void *data, const void *weight,

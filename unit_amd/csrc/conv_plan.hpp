@@ -13,13 +13,17 @@ struct TileShape {
   bool ff;                     // all fragments of a stage read at once (small wave tiles)
   int kg;                      // k-groups sharing the output tile
   bool direct;                 // operands straight from global memory to registers (int8 NCHW16c)
+  bool lds;                    // operand tiles shared through LDS by direct loads (prepared int8 NCHW16c weights only)
 };
 
 // index = variant id used by the tuning table and UNIT_AMD_CONV_VARIANT (1-based there)
 constexpr TileShape kConvTiles[] = {
-#define UNIT_CONV_VARIANT(ID, BX, BY, BKB, WX, WY, PF, FF, KG) {BX, BY, BKB, (WX) * (WY) * (KG), PF, FF, KG, false},
-#define UNIT_CONV_DIRECT(ID, TX, TY, KG, D) {(TX) * 32, (TY) * 32, 32, KG, (D) % 16, false, KG, true},
+#define UNIT_CONV_VARIANT(ID, BX, BY, BKB, WX, WY, PF, FF, KG) {BX, BY, BKB, (WX) * (WY) * (KG), PF, FF, KG, false, false},
+#define UNIT_CONV_DIRECT(ID, TX, TY, KG, D) {(TX) * 32, (TY) * 32, 32, KG, (D) % 16, false, KG, true, false},
+#define UNIT_CONV_LDS(ID, TX, TY, WX, WY, KG, KS, NST) \
+  {(TX) * (WX) * 32, (TY) * (WY) * 32, 32 * (KS), (WX) * (WY) * (KG), NST, false, KG, false, true},
 #include "conv_variants.def"
+#undef UNIT_CONV_LDS
 #undef UNIT_CONV_DIRECT
 #undef UNIT_CONV_VARIANT
 };
@@ -121,7 +125,7 @@ inline ConvPlan heuristic_plan(int npix, int K, int kbytes, bool allow_split, bo
 }
 
 inline ConvPlan plan_conv(const unit_conv_desc *d, int npix, int kbytes, const TunedConv *table, int ntable,
-                          bool allow_split, bool direct_ok, bool staged_too = false) {
+                          bool allow_split, bool direct_ok, bool staged_too = false, bool lds_ok = false) {
   ConvPlan p = heuristic_plan(npix, d->K, kbytes, allow_split, direct_ok, d->sh * d->sw > 1, staged_too);
   // UNIT_AMD_CONV_NOTABLE=1: heuristic only (the tuner measures it as the baseline)
   if (tuning_override("UNIT_AMD_CONV_NOTABLE") > 0) ntable = 0;
@@ -130,7 +134,8 @@ inline ConvPlan plan_conv(const unit_conv_desc *d, int npix, int kbytes, const T
     // the tables were tuned on square strides without dilation; a direct choice needs a window the direct
     // kernels can run, otherwise the heuristic's (staged) choice stands
     if (e.npix == npix && e.K == d->K && e.C == d->C && e.KH == d->KH && e.KW == d->KW && e.sh == d->sh &&
-        d->sw == d->sh && d->dh == 1 && d->dw == 1 && (direct_ok || !kConvTiles[e.variant].direct)) {
+        d->sw == d->sh && d->dh == 1 && d->dw == 1 && (direct_ok || !kConvTiles[e.variant].direct) &&
+        (lds_ok || !kConvTiles[e.variant].lds)) {
       p = ConvPlan{e.variant, e.splits, e.panel};
       break;
     }
@@ -148,6 +153,12 @@ inline ConvPlan plan_conv(const unit_conv_desc *d, int npix, int kbytes, const T
   const int op = tuning_override("UNIT_AMD_CONV_PANEL");
   if (op > 0) p.panel = op;
   if (!allow_split) p.splits = 1;
+  // the LDS-shared variants exist for prepared int8 weights only: elsewhere their ids run the heuristic's choice
+  if (kConvTiles[p.variant].lds && !lds_ok) {
+    const ConvPlan h = heuristic_plan(npix, d->K, kbytes, allow_split, direct_ok, d->sh * d->sw > 1, staged_too);
+    p.variant = h.variant;
+    if (!allow_split) p.splits = 1;
+  }
   return p;
 }
 

@@ -13,6 +13,13 @@ int conv_geom(const unit_conv_desc *d, int tapb, ConvGeom *g, const char *what);
 const TunedConv *tuned_conv_i8_prepared(int *n);                                  // below
 int conv_u8_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
                      const int *addend, void *out, hipStream_t s);  // conv_prepared_u8.hip
+int conv_u8_prepared_lds(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
+                         const char *zero, const int *addend, void *out, hipStream_t s);  // conv_lds_u8.hip
+int conv_s8_prepared_lds(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
+                         const char *zero, const int *bias, int scale, void *out, int planar, hipStream_t s);  // conv_lds_s8.hip
+int conv_q8_prepared_lds(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
+                         const char *zero, const int *addend, const int *bias, int scale, int shift, void *out,
+                         hipStream_t s);  // conv_lds_q8.hip
 int conv_s8_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
                      const int *bias, int scale, void *out, int planar, hipStream_t s);  // conv_prepared_s8.hip
 int conv_c4_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
@@ -60,8 +67,12 @@ __global__ __launch_bounds__(64) void prepare_i8_c4(const char *__restrict__ w, 
 // one wave per output channel: 128 * sum of its weights (a tap of a 16-output-channel block is
 // `dwords` dwords per channel, 64 bytes apart)
 __global__ __launch_bounds__(64) void prepare_i8_addend(const char *__restrict__ w, int *__restrict__ addend, int K,
-                                                        int ntaps, int dwords) {
+                                                        int ntaps, int dwords, int *__restrict__ zero_line) {
   const int ko = blockIdx.x, lane = threadIdx.x;
+  if (ko < 32) {  // the grid has 32 x kblocks >= 32 workgroups: each clears 1/32 of the zero region
+    constexpr int per = kZeroLine / 4 / 32;
+    for (int i = lane; i < per; i += 64) zero_line[ko * per + i] = 0;
+  }
   int sum = 0;
   if (ko < K) {
     const size_t tapb = (size_t)dwords * 64;
@@ -114,10 +125,13 @@ const TunedConv kTunedF16Prepared[] = {
 
 // Prepared weights exist for the direct kernels only: a table entry or override that names a
 // staged variant falls back to the heuristic's direct choice.
+// lds_ok: the entry point also has the LDS-shared kernels (int8, 16-channel blocks).
 ConvPlan plan_prepared(const unit_conv_desc *d, const ConvGeom &g, int kbytes, const TunedConv *table, int ntable,
-                       bool int8) {
-  ConvPlan p = plan_conv(d, g.npix, kbytes, table, ntable, int8, true);
-  if (!kConvTiles[p.variant].direct) p = heuristic_plan(g.npix, d->K, kbytes, int8, true, d->sh * d->sw > 1);
+                       bool int8, bool lds_ok = false) {
+  lds_ok = lds_ok && d->cb == 16;
+  ConvPlan p = plan_conv(d, g.npix, kbytes, table, ntable, int8, true, false, lds_ok);
+  const TileShape &t = kConvTiles[p.variant];
+  if (!(t.direct || (t.lds && lds_ok))) p = heuristic_plan(g.npix, d->K, kbytes, int8, true, d->sh * d->sw > 1);
   p.splits = 1;
   return p;
 }
@@ -171,7 +185,8 @@ extern "C" int unit_conv2d_prepare_weight(int32_t K, int32_t C, int32_t KH, int3
     else
       hipLaunchKernelGGL(prepare_i8, dim3(pl.kblocks * pl.nsteps), dim3(64), 0, s, w, out, K, ntaps, pl.nsteps);
     hipLaunchKernelGGL(prepare_i8_addend, dim3(pl.kblocks * 32), dim3(64), 0, s, w,
-                       reinterpret_cast<int *>(out + pl.frag_bytes), K, ntaps, cb / 4);
+                       reinterpret_cast<int *>(out + pl.frag_bytes), K, ntaps, cb / 4,
+                       reinterpret_cast<int *>(out + pl.zero_off));
   } else {
     hipLaunchKernelGGL(prepare_f16, dim3(pl.kblocks * pl.nsteps), dim3(64), 0, s, w, out, K, ntaps);
   }
@@ -195,11 +210,12 @@ extern "C" int unit_conv2d_nchwc_u8s8s32_prepared(const unit_conv_desc *d, const
   if (int rc = check_prepared_conv(what, d, 16, &g, data, prepared, out)) return rc;
   const PreparedLayout pl = prepared_layout(d->K, d->C, d->KH, d->KW, d->cb, 1);
   const int ntable = (int)(sizeof(kTunedI8Prepared) / sizeof(kTunedI8Prepared[0])) - 1;
-  const ConvPlan p = plan_prepared(d, g, g.ntaps * d->cb, kTunedI8Prepared, ntable, true);
+  const ConvPlan p = plan_prepared(d, g, g.ntaps * d->cb, kTunedI8Prepared, ntable, true, true);
   const char *w = static_cast<const char *>(prepared);
   const int *addend = reinterpret_cast<const int *>(w + pl.frag_bytes);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (d->cb == 4) return conv_c4_prepared(p, d, g, data, w, addend, 1, true, out, 0, s);
+  if (kConvTiles[p.variant].lds) return conv_u8_prepared_lds(p, d, g, data, w, w + pl.zero_off, addend, out, s);
   return conv_u8_prepared(p, d, g, data, w, addend, out, s);
 }
 
@@ -219,7 +235,7 @@ extern "C" int unit_conv2d_nchwc_u8s8u8_requant_prepared(const unit_conv_desc *d
   if (int rc = check_prepared_conv(what, d, 16, &g, data, prepared, out)) return rc;
   const PreparedLayout pl = prepared_layout(d->K, d->C, d->KH, d->KW, d->cb, 1);
   const int ntable = (int)(sizeof(kTunedI8Prepared) / sizeof(kTunedI8Prepared[0])) - 1;
-  const ConvPlan p = plan_prepared(d, g, g.ntaps * d->cb, kTunedI8Prepared, ntable, true);
+  const ConvPlan p = plan_prepared(d, g, g.ntaps * d->cb, kTunedI8Prepared, ntable, true, true);
   const char *w = static_cast<const char *>(prepared);
   // (v * scale + 2^(shift-1)) >> shift is unchanged when scale doubles and shift grows by one; with
   // shift >= 33 the kernel needs only the high dword of the product
@@ -227,6 +243,9 @@ extern "C" int unit_conv2d_nchwc_u8s8u8_requant_prepared(const unit_conv_desc *d
     scale *= 2;
     ++shift;
   }
+  if (kConvTiles[p.variant].lds)
+    return conv_q8_prepared_lds(p, d, g, data, w, w + pl.zero_off, reinterpret_cast<const int *>(w + pl.frag_bytes), bias,
+                                scale, shift, out, static_cast<hipStream_t>(stream));
   return conv_q8_prepared(p, d, g, data, w, reinterpret_cast<const int *>(w + pl.frag_bytes), bias, scale, shift, out,
                           static_cast<hipStream_t>(stream));
 }
@@ -248,9 +267,14 @@ int fused_prepared(const char *what, const unit_conv_desc *d, const void *data, 
   ConvGeom g;
   if (int rc = check_prepared_conv(what, d, 16, &g, data, prepared, out)) return rc;
   const int ntable = (int)(sizeof(kTunedI8Prepared) / sizeof(kTunedI8Prepared[0])) - 1;
-  const ConvPlan p = plan_prepared(d, g, g.ntaps * d->cb, kTunedI8Prepared, ntable, true);
+  const ConvPlan p = plan_prepared(d, g, g.ntaps * d->cb, kTunedI8Prepared, ntable, true, true);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (d->cb == 4) return conv_c4_prepared(p, d, g, data, prepared, bias, scale, false, out, planar, s);
+  if (kConvTiles[p.variant].lds) {
+    const PreparedLayout pl = prepared_layout(d->K, d->C, d->KH, d->KW, d->cb, 1);
+    return conv_s8_prepared_lds(p, d, g, data, prepared, static_cast<const char *>(prepared) + pl.zero_off, bias, scale,
+                                out, planar, s);
+  }
   return conv_s8_prepared(p, d, g, data, prepared, bias, scale, out, planar, s);
 }
 

@@ -9,7 +9,8 @@
 //     fp16: channel kb * 32 + lane % 32, tap s, input channels 8 (lane / 32) .. + 8;
 //   channels past K and the tap that pads an odd tap count are zeros;
 //   int8 only, behind the fragments: int32 addend[kb * 32 + c] = 128 * sum of the channel's weights
-//   (what a u8 convolution computed on x ^ 0x80 has to add back).
+//   (what a u8 convolution computed on x ^ 0x80 has to add back), then 16 KiB of zeros: the lines that the
+//   LDS-shared kernels (conv_lds.hpp) fetch in place of a tap that falls into the zero padding.
 #pragma once
 #include <cstddef>
 
@@ -18,8 +19,12 @@ namespace unit {
 struct PreparedLayout {
   int kblocks, nsteps;
   size_t frag_bytes;    // kblocks * nsteps * 1 KiB
-  size_t total_bytes;   // + the addends for int8
+  size_t total_bytes;   // + the addends and the zero line for int8
+  size_t zero_off;      // int8: byte offset of the zero line
 };
+// 16 KiB of zeros, not one line: every padded tap of every workgroup on the chip fetches from here, and a single
+// line would make one L2 channel the hot spot of the whole kernel; lanes pick a line by workgroup, wave and tap
+constexpr int kZeroLine = 16384;
 
 inline PreparedLayout prepared_layout(int K, int C, int KH, int KW, int cb, int elem_bytes) {
   PreparedLayout p;
@@ -27,7 +32,8 @@ inline PreparedLayout prepared_layout(int K, int C, int KH, int KW, int cb, int 
   p.kblocks = (K + 31) / 32;
   p.nsteps = cb == 4 ? (C / 4) * KH : (elem_bytes == 1 ? (ntaps + 1) / 2 : ntaps);
   p.frag_bytes = (size_t)p.kblocks * p.nsteps * 1024;
-  p.total_bytes = p.frag_bytes + (elem_bytes == 1 ? (size_t)p.kblocks * 32 * 4 : 0);
+  p.zero_off = p.frag_bytes + (size_t)p.kblocks * 32 * 4;
+  p.total_bytes = elem_bytes == 1 ? p.zero_off + kZeroLine : p.frag_bytes;
   return p;
 }
 
