@@ -77,7 +77,14 @@ def main():
                     help="launch one kernel 20 times and exit (for rocprofv3): a ResNet-50 layer name such as "
                          "3x3_256_256@14 (append :f16 for the fp16 convolution, :cold to cycle operand copies), "
                          "or gemm_i8 / gemm_f16 / gemm_f16_prepared / copy / pack_u8")
+    ap.add_argument("--profile-batch", type=int, default=None, metavar="N",
+                    help="batch of the --profile launches of a layer (default: the benchmark's 32)")
     args = ap.parse_args()
+    if args.profile_batch:
+        if not args.profile:
+            ap.error("--profile-batch goes with --profile")
+        global BATCH
+        BATCH = args.profile_batch
     if args.gpus != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus must be 1 "
               "(nothing here shards across devices)", file=sys.stderr)
