@@ -128,6 +128,16 @@ int unit_dense_dotprod_u8s8s32(const void *a, const void *wp, void *c, int32_t M
 int unit_dense_u8s8s32(const void *a, const void *w, void *c, int32_t M, int32_t N, int32_t K,
                        unit_stream_t stream);
 
+/* The same dense with the constant part of the u8 -> s8 shift folded once per weight, as the reference's
+ * compiled graphs fold sum(w) next to their u8 x s8 operators (apps/cpu/relay/result.log:15-16 for the
+ * convolution; the dense weight of apps/cpu/relay/int8-gemm.py:15 is a constant the same way):
+ *   unit_dense_prepare_weight  wsum[n] = sum_k w[n][k]  (int32[N], caller-owned)
+ *   unit_dense_u8s8s32_prepared  c = a . w^T with both operand tiles moved global -> LDS directly (K % 128 == 0
+ *   and at least 128 tiles of 256 x 256; other shapes run unit_dense_u8s8s32).  Results are identical. */
+int unit_dense_prepare_weight(const void *w, int32_t *wsum, int32_t N, int32_t K, unit_stream_t stream);
+int unit_dense_u8s8s32_prepared(const void *a, const void *w, const int32_t *wsum, void *c, int32_t M,
+                                int32_t N, int32_t K, unit_stream_t stream);
+
 /* ------------------------------------------------------------------ fp16 compute */
 
 /* The fp16 GEMM of apps/gpu/gemm.py:8-20 (CUDA form: poc/tensorcore/gemm-prefetch.cu:66-164):

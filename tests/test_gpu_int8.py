@@ -368,3 +368,31 @@ def test_full_size_properties(dev):
     o1 = U.conv2d_NCHWc_int8(_t(d1, dev), wt, 1, 1)
     o32 = U.conv2d_NCHWc_int8(_t(np.repeat(d1, 32, axis=0), dev), wt, 1, 1)
     assert torch.equal(o32, o1.expand(32, -1, -1, -1, -1))
+
+
+@pytest.mark.parametrize("M,N,K", [(512, 8192, 256), (4096, 4096, 128), (2000, 4100, 384), (64, 128, 128), (300, 4096, 144)])
+def test_dense_on_prepared_weight(dev, oracle, M, N, K):
+    """Weight sums folded once (unit_dense_prepare_weight): shapes with whole 128-byte stages and half a chip of
+    256 x 256 tiles run the direct-to-LDS kernel, ragged M / N included; the others fall back to the plain entry.
+    Bit-exact against a . W^T either way."""
+    a = rng.uniform_u8((M, K), 70 + M)
+    w = rng.uniform_s8((N, K), 71 + N)
+    p = U.prepare_dense_weight(_t(w, dev))
+    assert np.array_equal(p.wsum.cpu().numpy(), w.astype(np.int64).sum(axis=1))
+    out = U.dense(_t(a, dev), p)
+    torch.cuda.synchronize()
+    big = K % 128 == 0 and -(-M // 256) * -(-N // 256) >= 128
+    assert ("prep_dma" in U.last_variant()) == big, U.last_variant()
+    assert np.array_equal(out.cpu().numpy(), oracle.dense_logical(a, w)), U.last_variant()
+
+
+def test_dense_on_prepared_weight_extremes(dev, oracle):
+    """255 x -128 everywhere: the largest magnitudes the u8 shift and its correction see."""
+    M, N, K = 4096, 2048, 512
+    a = np.full((M, K), 255, np.uint8)
+    w = np.full((N, K), -128, np.int8)
+    w[::3] = 127
+    out = U.dense(_t(a, dev), U.prepare_dense_weight(_t(w, dev)))
+    torch.cuda.synchronize()
+    assert "prep_dma" in U.last_variant()
+    assert np.array_equal(out.cpu().numpy(), oracle.dense_logical(a, w))

@@ -169,7 +169,7 @@ def test_bench_final_line_fits_the_tail_budget():
                                     "number=3 each, mean x multiplicity",
                              seconds=0.044, gemm_int8_tops=17.61, gemm_fp16_tflops=1.31),
         "best_mfma_bound_layer": dict(layer="3x3_512_512@7", us=9.67, pct_int8_peak=15.2),
-        "gemm_int8_us": 80.39, "gemm_int8_pct_peak": 33.97, "gemm_fp16_us": 143.58, "gemm_fp16_tflops": 957.2,
+        "gemm_int8_us": 80.39, "gemm_int8_pct_peak": 33.97, "gemm_int8_prepared_w_us": 72.31, "gemm_int8_prepared_w_pct_peak": 37.77, "gemm_fp16_us": 143.58, "gemm_fp16_tflops": 957.2,
         "gemm_fp16_pct_peak": 38.05, "gemm_fp16_prepared_b_us": 119.64, "gemm_fp16_prepared_b_pct_peak": 45.66,
         "gemm_fp16_max_rel_err": 0.000247, "sum_layers_cold_us": 612.3, "launch": "hipgraph",
         "fp16_conv": dict(stack_us=618.2, tflops=387.0),

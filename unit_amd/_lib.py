@@ -22,6 +22,8 @@ SYMBOLS = (
     "unit_conv3d_ncdhwc_s8s8s32",
     "unit_dense_dotprod_u8s8s32",
     "unit_dense_u8s8s32",
+    "unit_dense_prepare_weight",
+    "unit_dense_u8s8s32_prepared",
     "unit_gemm_f16",
     "unit_gemm_f16_prepare_b",
     "unit_gemm_f16_prepare_b_packed32",
@@ -85,6 +87,8 @@ def load():
     L.unit_conv3d_ncdhwc_s8s8s32.argtypes = [ctypes.POINTER(Conv3dDesc), vp, vp, vp, vp]
     L.unit_dense_dotprod_u8s8s32.argtypes = [vp, vp, vp, i32, i32, i32, vp]
     L.unit_dense_u8s8s32.argtypes = [vp, vp, vp, i32, i32, i32, vp]
+    L.unit_dense_prepare_weight.argtypes = [vp, vp, i32, i32, vp]
+    L.unit_dense_u8s8s32_prepared.argtypes = [vp, vp, vp, vp, i32, i32, i32, vp]
     L.unit_gemm_f16.argtypes = [vp, vp, vp, i32, i32, i32, i32, vp]
     L.unit_gemm_f16_prepare_b.argtypes = [vp, vp, i32, i32, vp]
     L.unit_gemm_f16_prepare_b_packed32.argtypes = [vp, vp, i32, i32, vp]

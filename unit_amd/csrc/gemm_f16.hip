@@ -14,7 +14,7 @@ namespace {
 template <class T, int NSTAGE, bool OUT_F16>
 int run_gemm_f16_bt_dma(const void *a, const void *bt, void *c, int M, int N, int K, hipStream_t s) {
   using Epi = GemmEpilogue<OpF16, OUT_F16>;
-  DmaParams p{static_cast<const char *>(a), static_cast<const char *>(bt), M, N, K * 2};
+  DmaParams p{static_cast<const char *>(a), static_cast<const char *>(bt), M, N, K * 2, nullptr};
   typename Epi::Params ep{c, M, N};
   const int nk = K * 2 / T::BKB, gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
   constexpr int lds = NSTAGE * T::STAGE;
@@ -39,7 +39,7 @@ template <class T, bool OUT_F16>
 int run_gemm_f16_hybrid(const void *a, const void *b, void *c, int M, int N, int K, hipStream_t s) {
   using YL = KMajorF16Loader<T::BY, T::BKB, T::NT, 1, false>;
   using Epi = GemmEpilogue<OpF16, OUT_F16>;
-  DmaParams p{static_cast<const char *>(a), nullptr, M, N, K * 2};
+  DmaParams p{static_cast<const char *>(a), nullptr, M, N, K * 2, nullptr};
   typename YL::Params yp{static_cast<const char *>(b), N, K, N + 4, 0, N * 2};
   typename Epi::Params ep{c, M, N};
   const int nk = K * 2 / T::BKB, gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
@@ -64,7 +64,7 @@ template <class T, bool OUT_F16>
 int run_gemm_f16_bt_hybrid(const void *a, const void *bt, void *c, int M, int N, int K, hipStream_t s) {
   using YL = RowMajorLoader<T::BY, T::BKB, T::NT, false, 1, false>;
   using Epi = GemmEpilogue<OpF16, OUT_F16>;
-  DmaParams p{static_cast<const char *>(a), nullptr, M, N, K * 2};
+  DmaParams p{static_cast<const char *>(a), nullptr, M, N, K * 2, nullptr};
   typename YL::Params yp{static_cast<const char *>(bt), N, K * 2, K * 2};
   typename Epi::Params ep{c, M, N};
   const int nk = K * 2 / T::BKB, gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);

@@ -35,16 +35,17 @@ int run_dense(const void *a, const void *w, void *c, int M, int N, int K, hipStr
   }
 }
 
-// direct-to-LDS variant: row-major weights, K a whole number of stages
-template <class T, int NSTAGE>
-int run_dense_dma(const void *a, const void *w, void *c, int M, int N, int K, hipStream_t s) {
+// direct-to-LDS variant: row-major weights, K a whole number of stages.  wsum: the weight's row sums when they
+// were prepared beforehand (unit_dense_prepare_weight), else null and the kernel sums the fragments itself.
+template <class T, int NSTAGE, bool GIVEN = false>
+int run_dense_dma(const void *a, const void *w, void *c, int M, int N, int K, hipStream_t s, const int *wsum = nullptr) {
   using Epi = GemmEpilogue<OpI8, false>;
-  DmaParams p{static_cast<const char *>(a), static_cast<const char *>(w), M, N, K};
+  DmaParams p{static_cast<const char *>(a), static_cast<const char *>(w), M, N, K, wsum};
   typename Epi::Params ep{c, M, N};
   const int nk = K / T::BKB, gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
   constexpr int lds = NSTAGE * T::STAGE;
   static_assert(lds <= kMaxLds, "ring does not fit the LDS");
-  auto kern = mma_dma_kernel<OpI8, T, NSTAGE, Epi, WS_Y, true>;
+  auto kern = mma_dma_kernel<OpI8, T, NSTAGE, Epi, GIVEN ? WS_Y_GIVEN : WS_Y, true>;
   static thread_local bool allowed = false;
   if (!allowed) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -53,7 +54,7 @@ int run_dense_dma(const void *a, const void *w, void *c, int M, int N, int K, hi
     allowed = true;
   }
   GridMap gm{gx, gy, gx < 4 ? gx : 4, 1, gx * gy};
-  set_variant("i8densedma_x%d_y%d_k%d_w%d_r%d", T::BX, T::BY, T::BKB, T::NT / 64, NSTAGE);
+  set_variant("i8dense%sdma_x%d_y%d_k%d_w%dx%d_r%d", GIVEN ? "prep_" : "", T::BX, T::BY, T::BKB, T::WX, T::WY, NSTAGE);
   hipLaunchKernelGGL(kern, dim3(gm.total), dim3(T::NT), lds, s, p, ep, nk, gm);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "unit_dense_u8s8s32: launch: %s", hipGetErrorString(e));
@@ -128,8 +129,52 @@ int dense(const void *a, const void *w, void *c, int M, int N, int K, unit_strea
   return run_dense<Tile<128, 128, 64, 2, 2>, PACKED>(a, w, c, M, N, K, s);
 }
 
+// one wave per weight row: sum of its K bytes
+__global__ __launch_bounds__(256) void dense_row_sums(const char *__restrict__ w, int *__restrict__ sums, int N, int K) {
+  const int n = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (n >= N) return;
+  const int *row = reinterpret_cast<const int *>(w + (size_t)n * K);
+  int s = 0;
+  for (int i = lane; i < K / 4; i += 64) s = __builtin_amdgcn_sdot4(row[i], 0x01010101, s, false);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+  if (lane == 0) sums[n] = s;
+}
+
 }  // namespace
 }  // namespace unit
+
+extern "C" int unit_dense_prepare_weight(const void *w, int32_t *wsum, int32_t N, int32_t K, unit_stream_t stream) {
+  using namespace unit;
+  const char *what = "unit_dense_prepare_weight";
+  if (!w || !wsum) return fail(UNIT_E_ARG, "%s: null pointer", what);
+  if (N <= 0 || K <= 0 || K % 16) return fail(UNIT_E_ARG, "%s: N, K must be positive and K a multiple of 16 (got %d, %d)", what, N, K);
+  if (!fits((size_t)N * K)) return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
+  if (int rc = check_aligned(what, {w})) return rc;
+  if (int rc = check_device()) return rc;
+  hipLaunchKernelGGL(dense_row_sums, dim3(ceil_div(N, 4)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const char *>(w), wsum, N, K);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "%s: launch: %s", what, hipGetErrorString(e));
+  set_variant("dense_row_sums_n%d_k%d", N, K);
+  return UNIT_OK;
+}
+
+extern "C" int unit_dense_u8s8s32_prepared(const void *a, const void *w, const int32_t *wsum, void *c, int32_t M, int32_t N,
+                                           int32_t K, unit_stream_t stream) {
+  using namespace unit;
+  const char *what = "unit_dense_u8s8s32_prepared";
+  if (!a || !w || !wsum || !c) return fail(UNIT_E_ARG, "%s: null pointer", what);
+  // the direct-to-LDS kernel needs whole 128-byte stages and pays from half a chip of 256 x 256 tiles on;
+  // everything else runs the plain entry point, which sums the weights itself (same result)
+  const long tiles = (long)ceil_div(M, 256) * ceil_div(N, 256);
+  if (M <= 0 || N <= 0 || K <= 0 || K % 128 || N % 4 || tiles < 128 || row_slice(M, (size_t)K, (size_t)N * 4) ||
+      !fits((size_t)M * K) || !fits((size_t)N * K) || !fits((size_t)M * N * 4))
+    return unit_dense_u8s8s32(a, w, c, M, N, K, stream);
+  if (int rc = check_aligned(what, {a, w, c})) return rc;
+  if (int rc = check_device()) return rc;
+  return run_dense_dma<Tile<256, 256, 128, 4, 2>, 2, true>(a, w, c, M, N, K, static_cast<hipStream_t>(stream), wsum);
+}
 
 extern "C" int unit_dense_dotprod_u8s8s32(const void *a, const void *wp, void *c, int32_t M, int32_t N, int32_t K,
                                           unit_stream_t stream) {

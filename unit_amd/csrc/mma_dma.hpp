@@ -24,6 +24,7 @@ struct DmaParams {
   const char *y;  // Y rows
   int xrows, yrows;
   int ld;         // bytes per row (both operands)
+  const int *ysum;  // WS_Y_GIVEN: sum of each Y row's bytes (the int8 weight sums), computed once per weight
 };
 
 template <class Op, class T, int NSTAGE, class Epi, int WS, bool XOR_X>
@@ -147,7 +148,7 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
       __builtin_amdgcn_sched_barrier(0);
     }
   };
-  static_assert(T::TX * T::TY >= LPS && T::TX * T::TY >= T::TX + T::TY && T::TX * T::TY >= 4 * T::TY,
+  static_assert(T::TX * T::TY >= LPS && T::TX * T::TY >= T::TX + T::TY && (WS != WS_Y || T::TX * T::TY >= 4 * T::TY),
                 "not enough MFMAs per k-step to carry the step's other work");
 
   // One stage.  ISSUE: stage kt + NSTAGE exists and is fetched into the buffer this stage
@@ -196,6 +197,13 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
   if constexpr (WS == WS_Y) {
 #pragma unroll
     for (int j = 0; j < T::TY; ++j) wsy[j] += __shfl_xor(wsy[j], 32);
+  }
+  if constexpr (WS == WS_Y_GIVEN) {
+#pragma unroll
+    for (int j = 0; j < T::TY; ++j) {
+      const int n = y0 + wy * (T::TY * 32) + j * 32 + l32;
+      wsy[j] = n < p.yrows ? p.ysum[n] : 0;
+    }
   }
   Epi::template store<T>(ep, acc, wsx, wsy, x0 + wx * (T::TX * 32), y0 + wy * (T::TY * 32), lane, wave, lds,
                          gm.splits > 1);

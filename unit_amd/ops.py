@@ -19,7 +19,7 @@ from ._lib import ConvDesc, check
 
 __all__ = [
     "conv2d_NCHWc_int8", "dense_dotprod", "dense", "conv2d_NCHW16c_OHWI16o", "gemm_fp16",
-    "pack_nchwc", "unpack_nchwc", "prepack_conv_weight", "prepack_dense_weight",
+    "pack_nchwc", "unpack_nchwc", "prepack_conv_weight", "prepack_dense_weight", "prepare_dense_weight", "PreparedDenseWeight",
     "prepack_conv_weight_f16", "conv_out_hw", "last_variant",
     "PreparedConvWeight", "prepare_conv2d_weight", "PreparedGemmB", "prepare_gemm_b",
     "conv2d_NCHWc_int8_requant",
@@ -366,8 +366,38 @@ def dense_dotprod(data, weight, bias=None, out_dtype="int32"):
     return out
 
 
+class PreparedDenseWeight:
+    """A dense weight (N, K) s8 with its row sums, computed once by `prepare_dense_weight`: the constant part of the
+    u8 -> s8 shift, which the reference's compiled graphs fold the same way (apps/cpu/relay/result.log:15-16)."""
+
+    def __init__(self, w, wsum):
+        self.w, self.wsum = w, wsum
+        self.shape = tuple(w.shape)
+
+
+def prepare_dense_weight(weight):
+    """(N, K) s8 -> PreparedDenseWeight, accepted by `dense`."""
+    weight = _dev(weight, "weight", torch.int8, 2)
+    n, k = weight.shape
+    wsum = torch.empty((n,), dtype=torch.int32, device=weight.device)
+    check(_lib.load().unit_dense_prepare_weight(weight.data_ptr(), wsum.data_ptr(), n, k, _stream()))
+    return PreparedDenseWeight(weight, wsum)
+
+
 def dense(data, weight, out_dtype="int32"):
-    """relay.nn.dense(x u8 (M, K), w s8 (N, K)) -> i32 (M, N)."""
+    """relay.nn.dense(x u8 (M, K), w s8 (N, K)) -> i32 (M, N); `weight` may be a PreparedDenseWeight."""
+    if isinstance(weight, PreparedDenseWeight):
+        data = _dev(data, "data", torch.uint8, 2)
+        if out_dtype != "int32":
+            raise ValueError(f"out_dtype: only 'int32' is supported, got {out_dtype!r}")
+        m, k = data.shape
+        n, k2 = weight.shape
+        if k2 != k:
+            raise ValueError(f"weight: expected (N, {k}), got {weight.shape}")
+        out = torch.empty((m, n), dtype=torch.int32, device=data.device)
+        check(_lib.load().unit_dense_u8s8s32_prepared(data.data_ptr(), weight.w.data_ptr(), weight.wsum.data_ptr(),
+                                                      out.data_ptr(), m, n, k, _stream()))
+        return out
     weight = _dev(weight, "weight", torch.int8, 2)
     return dense_dotprod(data, weight, None, out_dtype)
 
