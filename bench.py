@@ -418,13 +418,23 @@ def main():
     us_r16 = time_us(lambda: _lib.check(L.unit_gemm_f16(rha.data_ptr(), rhb.data_ptr(), rhc.data_ptr(), 128, 768, 3072, 0, stream)),
                      50, bursts=3)
     v_r16 = U.last_variant()
+    # the same product with the k-splits' partial tiles in a workspace, added in split order (deterministic)
+    ws_bytes = ctypes.c_size_t()
+    _lib.check(L.unit_gemm_f16_ws_bytes(128, 768, 3072, ctypes.byref(ws_bytes)))
+    rws = torch.empty((max(ws_bytes.value, 16),), dtype=torch.uint8, device=dev)
+    rhc2 = torch.empty((128, 768), dtype=torch.float32, device=dev)
+    us_r16w = time_us(lambda: _lib.check(L.unit_gemm_f16_ws(rha.data_ptr(), rhb.data_ptr(), rhc2.data_ptr(), 128, 768, 3072, 0,
+                                                            rws.data_ptr(), rws.numel(), stream)), 50, bursts=3)
+    v_r16w = U.last_variant()
     torch.cuda.synchronize()
     want = rha.float() @ rhb.float()
     gemm_ref_sizes = dict(
         int8_dense_128x3072x768=dict(us=round(us_r8, 2), kernel=v_r8, source="apps/cpu/kernel/int8-gemm.py:9, apps/cpu/relay/int8-gemm.py:14-16"),
         fp16_gemm_128x768x3072=dict(us=round(us_r16, 2), kernel=v_r16, source="apps/gpu/gemm.py:6",
-                                    max_rel_err=float(((rhc - want).abs() / want.abs().clamp_min(1e-3 * float(want.abs().max()))).max())))
-    del ra, rw, rc, rha, rhb, rhc, want
+                                    max_rel_err=float(((rhc - want).abs() / want.abs().clamp_min(1e-3 * float(want.abs().max()))).max())),
+        fp16_gemm_128x768x3072_workspace=dict(us=round(us_r16w, 2), kernel=v_r16w, workspace_bytes=ws_bytes.value,
+                                              max_rel_err=float(((rhc2 - want).abs() / want.abs().clamp_min(1e-3 * float(want.abs().max()))).max())))
+    del ra, rw, rc, rha, rhb, rhc, rhc2, rws, want
     detail("gemm_int8_4096", **gemm_i8)
     detail("gemm_fp16_4096", **gemm_f16)
     detail("gemm_reference_sizes", **gemm_ref_sizes)

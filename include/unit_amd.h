@@ -152,6 +152,18 @@ int unit_dense_u8s8s32_prepared(const void *a, const void *w, const int32_t *wsu
 int unit_gemm_f16(const void *a, const void *b, void *c, int32_t M, int32_t N, int32_t K,
                   int32_t out_f16, unit_stream_t stream);
 
+/* The same GEMM with the k-splits' partial tiles kept apart: split s writes plane s (M * N floats) of a
+ * caller-owned workspace and a second kernel adds the planes in split order, as the reference's host
+ * check adds its split-K partial sums in a fixed order (poc/tensorcore/gemm-prefetch.cu:213-228).  The result no
+ * longer depends on which workgroup finishes first (bit-identical from run to run), and f16 output can use the
+ * k-splits too (the sum is rounded once).  unit_gemm_f16_ws_bytes gives the workspace size for a shape: 0 when
+ * the shape has enough output tiles, or too short a reduction, to run without k-splits (then workspace may be
+ * null and the call is unit_gemm_f16 with one workgroup per tile).  Same argument rules as unit_gemm_f16;
+ * M * N * 4 bytes <= 2^31 - 1. */
+int unit_gemm_f16_ws_bytes(int32_t M, int32_t N, int32_t K, size_t *bytes);
+int unit_gemm_f16_ws(const void *a, const void *b, void *c, int32_t M, int32_t N, int32_t K, int32_t out_f16,
+                     void *workspace, size_t workspace_bytes, unit_stream_t stream);
+
 /* _conv2d_NCHW16c_OHWI16o_impl(a, b, stride_h, stride_w, out_type)
  * (python/tensorizer/ops/gpu.py:8-53) on packed operands:
  *   a   f16 (N, C/16, H, W, 16)

@@ -215,3 +215,42 @@ def test_gemm_fp16_full_size(dev):
     rows = np.arange(0, M, 97)
     ref = a[rows].astype(np.float64) @ b.astype(np.float64)
     assert max_rel(out[rows], ref) <= REL_TOL
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 768, 3072), (256, 512, 8192), (100, 260, 1024), (512, 512, 256), (96, 64, 4096)])
+@pytest.mark.parametrize("out_dtype", ["float32", "float16"])
+def test_gemm_fp16_k_splits_through_a_workspace(dev, oracle, M, N, K, out_dtype):
+    """unit_gemm_f16_ws: partial tiles of the k-splits in planes of a workspace, added in split order.  Within the
+    1e-2 tolerance of float64 (2e-3 more for the final fp16 rounding), bit-identical from run to run, available
+    for fp16 output; a shape that needs no k-splits asks for no workspace and gives unit_gemm_f16's result."""
+    a = rng.normal_f16((M, K), 11 + M, 1.0 / np.sqrt(K))
+    b = rng.normal_f16((K, N), 12 + N)
+    ta, tb = _t(a, dev), _t(b, dev)
+    need = U.gemm_fp16_workspace_bytes(M, N, K)
+    ws = torch.full((need + 64,), 0xAB, dtype=torch.uint8, device=dev)  # stale contents must not matter
+    out1 = U.gemm_fp16(ta, tb, out_dtype, workspace=ws)
+    name = U.last_variant()
+    ws.fill_(0x5C)
+    out2 = U.gemm_fp16(ta, tb, out_dtype, workspace=ws)
+    torch.cuda.synchronize()
+    assert torch.equal(out1, out2), name
+    assert ("planes" in name) == (need > 0), (name, need)
+    ref = oracle.gemm_f16(a, b)
+    err = max_rel(out1.float().cpu().numpy(), ref)
+    assert err <= REL_TOL + (2e-3 if out_dtype == "float16" else 0), (err, name)
+    if need == 0:
+        assert torch.equal(out1, U.gemm_fp16(ta, tb, out_dtype)), name
+    else:
+        with pytest.raises(ValueError, match="workspace"):
+            U.gemm_fp16(ta, tb, out_dtype, workspace=ws[:need - 16])
+
+
+def test_gemm_fp16_workspace_integer_data_is_exact(dev, oracle):
+    """Integer-valued data: every partial sum is exact in fp32, so the planes add up to the float64 result bit for bit."""
+    M, N, K = 128, 768, 3072
+    a = (rng.uniform_u8((M, K), 5) % 7).astype(np.float16) - 3
+    b = (rng.uniform_u8((K, N), 6) % 5).astype(np.float16) - 2
+    out = U.gemm_fp16(_t(a, dev), _t(b, dev), "float32", workspace=True)
+    torch.cuda.synchronize()
+    assert "planes" in U.last_variant()
+    assert np.array_equal(out.cpu().numpy().astype(np.float64), oracle.gemm_f16(a, b))

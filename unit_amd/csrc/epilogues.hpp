@@ -11,6 +11,7 @@ namespace unit {
 // operand: out = acc + 128 * sum_k w[n][k].
 template <class Op, bool OUT_F16>
 struct GemmEpilogue {
+  static constexpr bool kSplitPlanes = false;
   struct Params {
     void *c;
     int M, N;
@@ -54,6 +55,28 @@ struct GemmEpilogue {
   }
 };
 
+// k-splits without atomics: split s of the fp16 GEMM writes its partial tile as plain fp32 stores into plane s of a
+// workspace (M * N floats each); a second kernel adds the planes in split order, so the result does not depend on
+// which workgroup finishes first, and can be rounded to fp16 afterwards.
+struct GemmPlaneEpilogue {
+  static constexpr bool kSplitPlanes = true;
+  struct Params {
+    void *c;  // plane 0 of the workspace
+    int M, N;
+    size_t plane;  // bytes per plane
+  };
+  template <class T>
+  static constexpr int lds_bytes() {
+    return 0;
+  }
+  template <class T>
+  static __device__ __forceinline__ void store(const Params &p, typename OpF16::acc_t (&acc)[T::TX][T::TY], int (&wsx)[T::TX],
+                                               int (&wsy)[T::TY], int xw0, int yw0, int lane, int wave, char *lds, int split) {
+    typename GemmEpilogue<OpF16, false>::Params q{static_cast<char *>(p.c) + (size_t)split * p.plane, p.M, p.N};
+    GemmEpilogue<OpF16, false>::template store<T>(q, acc, wsx, wsy, xw0, yw0, lane, wave, lds, false);
+  }
+};
+
 // Convolution output (N, K/16, OH, OW, 16), 4-byte elements: X rows are output channels, Y rows
 // are output pixels.  In the accumulators a lane holds one pixel and, per register quad, 4
 // consecutive channels; written like that, a store instruction would scatter 16-byte pieces over
@@ -65,6 +88,7 @@ struct GemmEpilogue {
 // the same per-wave LDS area once.
 template <class Op>
 struct ConvEpilogue {
+  static constexpr bool kSplitPlanes = false;
   struct Params {
     void *out;
     int K;     // output channels (multiple of 16)

@@ -197,8 +197,101 @@ int gemm_f16(const void *a, const void *b, void *c, int M, int N, int K, hipStre
   return run_gemm_f16<Tile<128, 128, 64, 2, 2>, OUT_F16>(a, b, c, M, N, K, s);
 }
 
+// ---- k-splits through a workspace: plane s of the workspace takes the partial tiles of split s, a second kernel
+// adds the planes in split order (deterministic; fp16 output rounds the final sum once)
+using SplitTile = Tile<128, 128, 64, 2, 2>;
+
+int gemm_f16_ws_splits(int M, int N, int K) {
+  return gemm_k_splits("UNIT_AMD_GEMM_F16_SPLITK", M, N, 2l * K, ceil_div(K * 2, SplitTile::BKB));
+}
+
+template <bool OUT_F16>
+__global__ __launch_bounds__(256) void add_planes(const v4f *__restrict__ ws, void *__restrict__ c, size_t n4, int splits,
+                                                  size_t plane4) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n4) return;
+  v4f sum = ws[i];
+  for (int s = 1; s < splits; ++s) sum += ws[i + s * plane4];
+  if constexpr (OUT_F16) {
+    typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+    static_cast<v4h *>(c)[i] = v4h{(_Float16)sum[0], (_Float16)sum[1], (_Float16)sum[2], (_Float16)sum[3]};
+  } else {
+    static_cast<v4f *>(c)[i] = sum;
+  }
+}
+
+// a (M, K) . b (K, N) with `splits` > 1 k-ranges; ws holds splits * M * N floats
+int gemm_f16_planes(const char *what, const void *a, const void *b, void *c, int M, int N, int K, bool out_f16, void *ws,
+                    int splits, hipStream_t s) {
+  using T = SplitTile;
+  using XL = RowMajorLoader<T::BX, T::BKB, T::NT, false, 1, true>;
+  using YL = KMajorF16Loader<T::BY, T::BKB, T::NT, 1, true>;
+  typename XL::Params xp{static_cast<const char *>(a), M, K * 2, K * 2};
+  typename YL::Params yp{static_cast<const char *>(b), N, K, N + 4, 0, N * 2};
+  const size_t plane = (size_t)M * N * 4;
+  GemmPlaneEpilogue::Params ep{ws, M, N, plane};
+  const int nk = ceil_div(K * 2, T::BKB), gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
+  set_variant("f16gemm_planes_x%d_y%d_k%d_w%dx%d%s_s%d", T::BX, T::BY, T::BKB, T::WX, T::WY, out_f16 ? "_h" : "", splits);
+  if (int rc = launch_mma<OpF16, T, XL, YL, GemmPlaneEpilogue, WS_NONE>(xp, yp, ep, nk, gx, gy, 4, splits, nullptr, 0, 0, s, what))
+    return rc;
+  const size_t n4 = (size_t)M * N / 4;
+  if (out_f16)
+    hipLaunchKernelGGL(add_planes<true>, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s, static_cast<const v4f *>(ws), c,
+                       n4, splits, n4);
+  else
+    hipLaunchKernelGGL(add_planes<false>, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s, static_cast<const v4f *>(ws),
+                       c, n4, splits, n4);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "%s: launch: %s", what, hipGetErrorString(e));
+}
+
+// argument checks shared by the entry points that split the reduction through planes; *splits = 1 when the shape
+// runs without k-splits (then the plain entry point serves it)
+int gemm_f16_ws_check(const char *what, const void *a, const void *b, const void *c, int M, int N, int K, int *splits) {
+  if (!a || !b || !c) return fail(UNIT_E_ARG, "%s: null pointer", what);
+  if (M <= 0 || N <= 0 || K <= 0) return fail(UNIT_E_ARG, "%s: M, N, K must be positive (got %d, %d, %d)", what, M, N, K);
+  if (K % 8) return fail(UNIT_E_ARG, "%s: K must be a multiple of 8 (got %d)", what, K);
+  if (N % 4) return fail(UNIT_E_ARG, "%s: N must be a multiple of 4 (got %d)", what, N);
+  if (!fits((size_t)M * K * 2) || !fits((size_t)N * K * 2) || !fits((size_t)M * N * 4))
+    return fail(UNIT_E_ARG, "%s: tensor exceeds 2^31-1 bytes", what);
+  *splits = gemm_f16_ws_splits(M, N, K);
+  return UNIT_OK;
+}
+
 }  // namespace
 }  // namespace unit
+
+extern "C" int unit_gemm_f16_ws_bytes(int32_t M, int32_t N, int32_t K, size_t *bytes) {
+  using namespace unit;
+  const char *what = "unit_gemm_f16_ws_bytes";
+  if (!bytes) return fail(UNIT_E_ARG, "%s: null pointer", what);
+  if (M <= 0 || N <= 0 || K <= 0 || K % 8 || N % 4)
+    return fail(UNIT_E_ARG, "%s: M, N, K must be positive, K a multiple of 8 and N of 4 (got %d, %d, %d)", what, M, N, K);
+  const int splits = gemm_f16_ws_splits(M, N, K);
+  *bytes = splits > 1 ? (size_t)splits * M * N * 4 : 0;
+  return UNIT_OK;
+}
+
+extern "C" int unit_gemm_f16_ws(const void *a, const void *b, void *c, int32_t M, int32_t N, int32_t K, int32_t out_f16,
+                                void *workspace, size_t workspace_bytes, unit_stream_t stream) {
+  using namespace unit;
+  const char *what = "unit_gemm_f16_ws";
+  int splits = 1;
+  if (int rc = gemm_f16_ws_check(what, a, b, c, M, N, K, &splits)) return rc;
+  if (splits <= 1) {  // enough tiles, or a short reduction: nothing to split (the plain path makes the same choice)
+    if (int rc = check_aligned(what, {a, b, c})) return rc;
+    if (int rc = check_device()) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return out_f16 ? gemm_f16<true>(a, b, c, M, N, K, s) : gemm_f16<false>(a, b, c, M, N, K, s);
+  }
+  const size_t need = (size_t)splits * M * N * 4;
+  if (!workspace || workspace_bytes < need)
+    return fail(UNIT_E_ARG, "%s: workspace of %zu bytes needed (got %zu); ask unit_gemm_f16_ws_bytes", what, need,
+                workspace ? workspace_bytes : (size_t)0);
+  if (int rc = check_aligned(what, {a, b, c, workspace})) return rc;
+  if (int rc = check_device()) return rc;
+  return gemm_f16_planes(what, a, b, c, M, N, K, out_f16 != 0, workspace, splits, static_cast<hipStream_t>(stream));
+}
 
 extern "C" int unit_gemm_f16(const void *a, const void *b, void *c, int32_t M, int32_t N, int32_t K,
                              int32_t out_f16, unit_stream_t stream) {

@@ -143,7 +143,7 @@ int launch_mma(const typename XL::Params &xp, const typename YL::Params &yp, con
   }
   if (splits < 1) splits = 1;
   if (splits > nk) splits = nk;
-  if (splits > 1) {
+  if (splits > 1 && !Epi::kSplitPlanes) {
     const size_t n16 = out_bytes / 16;
     hipLaunchKernelGGL(zero_fill, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, stream,
                        static_cast<v4i *>(out), n16);

@@ -390,8 +390,11 @@ __global__ __launch_bounds__(T::NT) void mma_kernel(typename XL::Params xp, type
   }
 
   // the last barrier of the K loop came after every LDS read: the tiles are free for the epilogue
-  Epi::template store<T>(ep, acc, wsx, wsy, x0 + wx * (T::TX * 32), y0 + wy * (T::TY * 32), lane, wave,
-                         lds, gm.splits > 1);
+  if constexpr (Epi::kSplitPlanes)  // every k-split writes a plane of its own: the last argument is the split
+    Epi::template store<T>(ep, acc, wsx, wsy, x0 + wx * (T::TX * 32), y0 + wy * (T::TY * 32), lane, wave, lds, split);
+  else
+    Epi::template store<T>(ep, acc, wsx, wsy, x0 + wx * (T::TX * 32), y0 + wy * (T::TY * 32), lane, wave, lds,
+                           gm.splits > 1);
 }
 
 // zero fill for outputs accumulated with atomics (k-splits): 16 bytes per thread

@@ -10,6 +10,7 @@ Reference call sites:
   conv2d_NCHW16c_OHWI16o   python/tensorizer/ops/gpu.py:8-53  (_conv2d_NCHW16c_OHWI16o_impl)
   gemm_fp16                apps/gpu/gemm.py:8-20
 """
+import ctypes
 import re
 
 import torch
@@ -18,7 +19,7 @@ from . import _lib
 from ._lib import ConvDesc, check
 
 __all__ = [
-    "conv2d_NCHWc_int8", "dense_dotprod", "dense", "conv2d_NCHW16c_OHWI16o", "gemm_fp16",
+    "conv2d_NCHWc_int8", "dense_dotprod", "dense", "conv2d_NCHW16c_OHWI16o", "gemm_fp16", "gemm_fp16_workspace_bytes",
     "pack_nchwc", "unpack_nchwc", "prepack_conv_weight", "prepack_dense_weight", "prepare_dense_weight", "PreparedDenseWeight",
     "prepack_conv_weight_f16", "conv_out_hw", "last_variant",
     "PreparedConvWeight", "prepare_conv2d_weight", "PreparedGemmB", "prepare_gemm_b",
@@ -432,10 +433,12 @@ def prepare_gemm_b(b):
     return PreparedGemmB(bt, k, n)
 
 
-def gemm_fp16(a, b, out_dtype="float32"):
+def gemm_fp16(a, b, out_dtype="float32", workspace=None):
     """c[x, y] = sum_k f32(a[x, k]) * f32(b[k, y]); a (M, K), b (K, N) fp16 row-major, or b a
     PreparedGemmB, or b packed (N/32, K/32, 32, 32) with b4[y/32][k/32][k%32][y%32] = b[k][y] as
-    apps/gpu/gemm-pack.py:9,14-18 takes it (re-laid on every call: prepare it once instead)."""
+    apps/gpu/gemm-pack.py:9,14-18 takes it (re-laid on every call: prepare it once instead).
+    workspace (b (K, N) only): True, or a uint8 tensor of `gemm_fp16_workspace_bytes(M, N, K)` bytes: k-splits keep
+    their partial tiles in it and are added in split order (run-to-run identical results, also for float16 output)."""
     a = _dev(a, "a", torch.float16, 2)
     if out_dtype not in ("float32", "float16"):
         raise ValueError(f"out_dtype: expected 'float32' or 'float16', got {out_dtype!r}")
@@ -455,8 +458,23 @@ def gemm_fp16(a, b, out_dtype="float32"):
     if k2 != k:
         raise ValueError(f"b: expected ({k}, N), got {tuple(b.shape)}")
     out = torch.empty((m, n), dtype=torch.float16 if half else torch.float32, device=a.device)
+    if workspace is not None and workspace is not False:
+        need = gemm_fp16_workspace_bytes(m, n, k)
+        if workspace is True:
+            workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=a.device)
+        workspace = _dev(workspace, "workspace", torch.uint8)
+        check(_lib.load().unit_gemm_f16_ws(a.data_ptr(), b.data_ptr(), out.data_ptr(), m, n, k, int(half),
+                                           workspace.data_ptr(), workspace.numel(), _stream()))
+        return out
     check(_lib.load().unit_gemm_f16(a.data_ptr(), b.data_ptr(), out.data_ptr(), m, n, k, int(half), _stream()))
     return out
+
+
+def gemm_fp16_workspace_bytes(m, n, k):
+    """Bytes `gemm_fp16(..., workspace=...)` needs for this shape (0: the shape runs without k-splits)."""
+    nbytes = ctypes.c_size_t()
+    check(_lib.load().unit_gemm_f16_ws_bytes(m, n, k, ctypes.byref(nbytes)))
+    return nbytes.value
 
 
 def conv2d_NCHW16c_OHWI16o(a, b, stride_h, stride_w, out_type="float32"):
