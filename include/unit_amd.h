@@ -164,6 +164,17 @@ int unit_gemm_f16_ws_bytes(int32_t M, int32_t N, int32_t K, size_t *bytes);
 int unit_gemm_f16_ws(const void *a, const void *b, void *c, int32_t M, int32_t N, int32_t K, int32_t out_f16,
                      void *workspace, size_t workspace_bytes, unit_stream_t stream);
 
+/* unit_gemm_f16_ws without the workspace argument: the planes live in a 16 MiB device array inside the library, so
+ * the call allocates nothing (no hipMalloc / hipFree, here or in anything it calls).  It has no counterpart in the
+ * reference; it is for callers that cannot allocate: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid allocation.  Same results as unit_gemm_f16_ws, bit for bit.  Shapes whose k-splits need more than
+ * 16 MiB (splits x M x N x 4 bytes; ask unit_gemm_f16_ws_bytes) are rejected with UNIT_E_ARG: pass a workspace to
+ * unit_gemm_f16_ws instead.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two
+ * streams, two threads) race, calls in stream order do not.  The first call on a device resolves the array's
+ * address there; make it outside graph capture. */
+int unit_gemm_f16_static(const void *a, const void *b, void *c, int32_t M, int32_t N, int32_t K, int32_t out_f16,
+                         unit_stream_t stream);
+
 /* _conv2d_NCHW16c_OHWI16o_impl(a, b, stride_h, stride_w, out_type)
  * (python/tensorizer/ops/gpu.py:8-53) on packed operands:
  *   a   f16 (N, C/16, H, W, 16)

@@ -27,6 +27,7 @@ SYMBOLS = (
     "unit_gemm_f16",
     "unit_gemm_f16_ws_bytes",
     "unit_gemm_f16_ws",
+    "unit_gemm_f16_static",
     "unit_gemm_f16_prepare_b",
     "unit_gemm_f16_prepare_b_packed32",
     "unit_gemm_f16_prepared",
@@ -92,6 +93,7 @@ def load():
     L.unit_dense_prepare_weight.argtypes = [vp, vp, i32, i32, vp]
     L.unit_gemm_f16_ws_bytes.argtypes = [i32, i32, i32, ctypes.POINTER(ctypes.c_size_t)]
     L.unit_gemm_f16_ws.argtypes = [vp, vp, vp, i32, i32, i32, i32, vp, ctypes.c_size_t, vp]
+    L.unit_gemm_f16_static.argtypes = [vp, vp, vp, i32, i32, i32, i32, vp]
     L.unit_dense_u8s8s32_prepared.argtypes = [vp, vp, vp, vp, i32, i32, i32, vp]
     L.unit_gemm_f16.argtypes = [vp, vp, vp, i32, i32, i32, i32, vp]
     L.unit_gemm_f16_prepare_b.argtypes = [vp, vp, i32, i32, vp]

@@ -1,5 +1,7 @@
 // fp16 GEMM: c (M, N) = a (M, K) f16 . b (K, N) f16, fp32 accumulate on v_mfma_f32_32x32x16_f16.
 // X operand = a (rows m, K-contiguous), Y operand = b (rows n, transposed while staging).
+#include <mutex>
+
 #include "epilogues.hpp"
 #include "host.hpp"
 #include "loaders.hpp"
@@ -260,6 +262,57 @@ int gemm_f16_ws_check(const char *what, const void *a, const void *b, const void
 
 }  // namespace
 }  // namespace unit
+
+// ---- the same planes in a buffer the library owns: a file-scope device array, so that the entry point below
+// allocates nothing.  Each GPU the library runs on holds its own copy of the array at its own address, resolved once
+// per device on the first call there (with that device current); host code uses that pointer, never the array's name.
+namespace unit {
+namespace {
+constexpr size_t kStaticScratchBytes = 16u << 20;
+static __device__ __align__(256) char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+void *g_scratch_ptr[kMaxDevices];
+std::mutex g_scratch_mutex;
+
+int static_scratch(const char *what, void **ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(UNIT_E_DEVICE, "%s: hipGetDevice: %s", what, hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(UNIT_E_DEVICE, "%s: device index %d out of range", what, dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void *p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr)
+      return fail(UNIT_E_DEVICE, "%s: hipGetSymbolAddress: %s", what, hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return UNIT_OK;
+}
+}  // namespace
+}  // namespace unit
+
+extern "C" int unit_gemm_f16_static(const void *a, const void *b, void *c, int32_t M, int32_t N, int32_t K, int32_t out_f16,
+                                    unit_stream_t stream) {
+  using namespace unit;
+  const char *what = "unit_gemm_f16_static";
+  int splits = 1;
+  if (int rc = gemm_f16_ws_check(what, a, b, c, M, N, K, &splits)) return rc;
+  if (int rc = check_aligned(what, {a, b, c})) return rc;
+  if (int rc = check_device()) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (splits <= 1)  // nothing to split: no scratch is touched
+    return out_f16 ? gemm_f16<true>(a, b, c, M, N, K, s) : gemm_f16<false>(a, b, c, M, N, K, s);
+  const size_t need = (size_t)splits * M * N * 4;
+  if (need > kStaticScratchBytes)
+    return fail(UNIT_E_ARG, "%s: %d k-splits of %d x %d need %zu bytes of scratch, the static buffer holds %zu; "
+                "use unit_gemm_f16_ws with a workspace", what, splits, M, N, need, kStaticScratchBytes);
+  void *ws = nullptr;
+  if (int rc = static_scratch(what, &ws)) return rc;
+  // every plane element that add_planes reads is written by this call's GEMM first: nothing has to start at zero
+  return gemm_f16_planes(what, a, b, c, M, N, K, out_f16 != 0, ws, splits, s);
+}
 
 extern "C" int unit_gemm_f16_ws_bytes(int32_t M, int32_t N, int32_t K, size_t *bytes) {
   using namespace unit;
