@@ -35,8 +35,9 @@ def test_mfma_tile_f16_lane_layout(dev):
 
 
 GEMM_CASES = [(128, 768, 3072), (32, 32, 64), (100, 132, 72), (512, 4096, 256), (4096, 2048, 512), (2050, 4100, 136),
-              (1024, 4096, 128), (1000, 4100, 192),  # 256 x 128 tiles of the hybrid pipeline, whole and ragged
-              (2050, 4100, 192)]                     # 256 x 256 tiles, ragged
+              (1024, 4096, 128), (300, 264, 96),     # both operands straight into LDS, 128 x 128 tiles, whole and ragged
+              (2050, 4104, 192), (2050, 4104, 160),  # the same on 256 x 256 tiles, 128- and 64-byte stages, ragged
+              (1000, 4100, 192), (2050, 4100, 192)]  # N not a multiple of 8: b through the transposing register loader
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_CASES)
@@ -97,11 +98,14 @@ def test_gemm_fp16_prepared_b_integer_exact(dev, oracle):
     M, N, K = 512, 768, 1024
     a = (np.arange(M * K).reshape(M, K) % 7).astype(np.float16)
     b = (np.arange(K * N).reshape(K, N) % 5 - 2).astype(np.float16)
-    for (m, n), kernel in (((M, N), "f16gemmbt_x"), ((4096, 2048), "hybrid_x256_y128"), ((4096, 4096), "dma_x256_y256")):
-        aa = np.resize(a, (m, K)); bb = np.resize(b, (K, n))
+    # 128 x 128 tiles with both operands straight into LDS, in two k-splits and whole; 256 x 256 tiles; and, with a
+    # reduction that is no whole number of 64-byte stages, the register pipeline
+    for (m, n, k), kernel in (((M, N, K), "dma_x128_y128_k64_w2x2_r4_s2"), ((4096, 2048, K), "dma_x128_y128_k64_w2x2_r4_s1"),
+                              ((4096, 4096, K), "dma_x256_y256"), ((M, N, 1000), "f16gemmbt_x")):
+        aa = np.resize(a, (m, k)); bb = np.resize(b, (k, n))
         out = U.gemm_fp16(_t(aa, dev), U.prepare_gemm_b(_t(bb, dev))).cpu().numpy()
         assert np.array_equal(out.astype(np.float64), oracle.gemm_f16(aa, bb)), U.last_variant()
-        assert kernel in U.last_variant(), U.last_variant()  # registers; 256 x 128 hybrid; 256 x 256 all direct-to-LDS
+        assert kernel in U.last_variant(), U.last_variant()
 
 
 @pytest.mark.parametrize("M,N,K", [(64, 192, 1024), (128, 768, 3072), (300, 2080, 96), (4096, 4096, 512)])
@@ -131,8 +135,15 @@ def test_gemm_fp16_integer_exact(dev, oracle):
     M, N, K = 256, 384, 512
     a = (np.arange(M * K).reshape(M, K) % 7).astype(np.float16)
     b = (np.arange(K * N).reshape(K, N) % 5 - 2).astype(np.float16)
-    out = U.gemm_fp16(_t(a, dev), _t(b, dev)).cpu().numpy()
-    assert np.array_equal(out.astype(np.float64), oracle.gemm_f16(a, b))
+    # b read back from LDS with the transposing read, on 128 x 128 tiles (k-splits and whole) and 256 x 256 tiles; N not
+    # a multiple of 8: b transposed in registers; K no whole number of stages: both operands through registers
+    for (m, n, k), kernel in (((M, N, K), "dmatr_x128_y128_k64_w2x2_r4_s4"), ((4096, 2048, K), "dmatr_x128_y128_k64_w2x2_r4_s1"),
+                              ((4096, 4096, K), "dmatr_x256_y256_k128"), ((4096, 4096, 96), "dmatr_x256_y256_k64"),
+                              ((2048, 2052, K), "hybrid_x256"), ((M, N, 1000), "f16gemm_x")):
+        aa = np.resize(a, (m, k)); bb = np.resize(b, (k, n))
+        out = U.gemm_fp16(_t(aa, dev), _t(bb, dev)).cpu().numpy()
+        assert np.array_equal(out.astype(np.float64), oracle.gemm_f16(aa, bb)), U.last_variant()
+        assert kernel in U.last_variant(), U.last_variant()
 
 
 CONV_CASES = [

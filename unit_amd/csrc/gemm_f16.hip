@@ -10,11 +10,35 @@
 namespace unit {
 namespace {
 
+// Which all-direct tile: 256 x 256 (eight waves, one workgroup per CU, the least LDS traffic per MFMA) or 128 x 128
+// (four waves, two workgroups per CU).  Measured time per 1024 of K: a round of large tiles 30 us (24 when under 200
+// CUs are busy), a round of 512 small tiles 21.5 us, 13 us when at most 256 are left (one per CU).
+inline bool gemm_f16_large_tiles(int M, int N) {
+  const long tb = (long)ceil_div(M, 256) * ceil_div(N, 256), t128 = (long)ceil_div(M, 128) * ceil_div(N, 128);
+  const double big = (double)((tb + 255) / 256) * (tb <= 200 ? 24.0 : 30.0);
+  const long rest = t128 % 512;
+  const double small = (double)(t128 / 512) * 21.5 + (rest == 0 ? 0.0 : rest <= 256 ? 13.0 : 21.5);
+  return M >= 256 && N >= 256 && big < small;
+}
+
+// k-splits of the 128 x 128 all-direct tiles (f32 output, added with atomics): up to 128 workgroups, and a split's
+// share of K at least 16 x the tile count (the zero fill and the atomics cost in proportion to the output: 1024^3 on
+// 64 tiles runs 14.5 us whole and 15.6 us in two splits, 512 x 512 x 4096 on 16 tiles 35 us whole and 15 us in 8)
+inline int gemm_f16_direct_splits(int M, int N, int K) {
+  int splits = tuning_override("UNIT_AMD_GEMM_F16_SPLITK");
+  if (splits <= 0) {
+    const long t128 = (long)ceil_div(M, 128) * ceil_div(N, 128);
+    const long share = 16 * t128 > 128 ? 16 * t128 : 128;
+    splits = (int)(128 / t128 < K / share ? 128 / t128 : K / share);
+  }
+  return splits < 1 ? 1 : splits;
+}
+
 // Prepared b: (N, K) rows, K-contiguous like a.  Both operands then go global -> LDS directly
 // (no register round trip, no transposition), through a ring of NSTAGE LDS buffers; K a whole
 // number of stages.
 template <class T, int NSTAGE, bool OUT_F16>
-int run_gemm_f16_bt_dma(const void *a, const void *bt, void *c, int M, int N, int K, hipStream_t s) {
+int run_gemm_f16_bt_dma(const void *a, const void *bt, void *c, int M, int N, int K, hipStream_t s, int splits = 1) {
   using Epi = GemmEpilogue<OpF16, OUT_F16>;
   DmaParams p{static_cast<const char *>(a), static_cast<const char *>(bt), M, N, K * 2, nullptr};
   typename Epi::Params ep{c, M, N};
@@ -28,15 +52,57 @@ int run_gemm_f16_bt_dma(const void *a, const void *bt, void *c, int M, int N, in
     if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "unit_gemm_f16_prepared: hipFuncSetAttribute: %s", hipGetErrorString(e));
     allowed = true;
   }
-  GridMap gm{gx, gy, gx < 4 ? gx : 4, 1, gx * gy};
-  set_variant("f16gemmbt_dma_x%d_y%d_k%d_w%dx%d_r%d%s", T::BX, T::BY, T::BKB, T::WX, T::WY, NSTAGE, OUT_F16 ? "_h" : "");
+  splits = OUT_F16 || splits < 1 ? 1 : (splits > nk ? nk : splits);
+  if (splits > 1) {  // the k-ranges add into c with atomics
+    const size_t n16 = (size_t)M * N * 4 / 16;
+    hipLaunchKernelGGL(zero_fill, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, s, static_cast<v4i *>(c), n16);
+  }
+  GridMap gm{gx, gy, gx < 4 ? gx : 4, splits, gx * gy * splits};
+  set_variant("f16gemmbt_dma_x%d_y%d_k%d_w%dx%d_r%d%s_s%d", T::BX, T::BY, T::BKB, T::WX, T::WY, NSTAGE, OUT_F16 ? "_h" : "",
+              splits);
   hipLaunchKernelGGL(kern, dim3(gm.total), dim3(T::NT), lds, s, p, ep, nk, gm);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "unit_gemm_f16_prepared: launch: %s", hipGetErrorString(e));
 }
 
-// b (K, N) as the reference gives it: a goes global -> LDS directly, b through the transposing
-// register loader (K a whole number of stages)
+// b (K, N) as the reference gives it, both operands global -> LDS directly: b's tile lands as it lies in memory and
+// the fragments come out of it with the LDS transposing read (K a whole number of stages, N a multiple of 8).
+// splits > 1: k-ranges, added with atomics into the zero-filled c (Epi = GemmEpilogue, f32) or written as planes.
+template <class T, int NSTAGE, class Epi>
+int run_gemm_f16_dma_tr(const char *what, const char *tag, const void *a, const void *b, const typename Epi::Params &ep,
+                        int M, int N, int K, int splits, void *zero, hipStream_t s) {
+  DmaParams p{static_cast<const char *>(a), static_cast<const char *>(b), M, N, K * 2, nullptr, N * 2};
+  const int nk = K * 2 / T::BKB, gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
+  constexpr int lds = NSTAGE * T::STAGE;
+  static_assert(lds <= kMaxLds, "ring does not fit the LDS");
+  auto kern = mma_dma_kernel<OpF16, T, NSTAGE, Epi, WS_NONE, false, true>;
+  static thread_local bool allowed = false;
+  if (!allowed) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
+    if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "%s: hipFuncSetAttribute: %s", what, hipGetErrorString(e));
+    allowed = true;
+  }
+  splits = splits < 1 ? 1 : (splits > nk ? nk : splits);
+  if (splits > 1 && zero) {
+    const size_t n16 = (size_t)M * N * 4 / 16;
+    hipLaunchKernelGGL(zero_fill, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, s, static_cast<v4i *>(zero), n16);
+  }
+  GridMap gm{gx, gy, gx < 4 ? gx : 4, splits, gx * gy * splits};
+  set_variant("f16gemm_%s_x%d_y%d_k%d_w%dx%d_r%d_s%d", tag, T::BX, T::BY, T::BKB, T::WX, T::WY, NSTAGE, splits);
+  hipLaunchKernelGGL(kern, dim3(gm.total), dim3(T::NT), lds, s, p, ep, nk, gm);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "%s: launch: %s", what, hipGetErrorString(e));
+}
+
+template <class T, int NSTAGE, bool OUT_F16>
+int run_gemm_f16_dma_tr(const void *a, const void *b, void *c, int M, int N, int K, hipStream_t s, int splits = 1) {
+  using Epi = GemmEpilogue<OpF16, OUT_F16>;
+  typename Epi::Params ep{c, M, N};
+  return run_gemm_f16_dma_tr<T, NSTAGE, Epi>("unit_gemm_f16", OUT_F16 ? "dmatr_h" : "dmatr", a, b, ep, M, N, K,
+                                             OUT_F16 ? 1 : splits, c, s);
+}
+
+// b (K, N): a goes global -> LDS directly, b through the transposing register loader (K a whole number of stages)
 template <class T, bool OUT_F16>
 int run_gemm_f16_hybrid(const void *a, const void *b, void *c, int M, int N, int K, hipStream_t s) {
   using YL = KMajorF16Loader<T::BY, T::BKB, T::NT, 1, false>;
@@ -60,31 +126,6 @@ int run_gemm_f16_hybrid(const void *a, const void *b, void *c, int M, int N, int
   return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "unit_gemm_f16: launch: %s", hipGetErrorString(e));
 }
 
-// prepared b (N, K) with a straight into LDS and b through the (non-transposing) register loader: the tile shapes the
-// all-direct kernel cannot carry (too few MFMAs per k-step for its waits)
-template <class T, bool OUT_F16>
-int run_gemm_f16_bt_hybrid(const void *a, const void *bt, void *c, int M, int N, int K, hipStream_t s) {
-  using YL = RowMajorLoader<T::BY, T::BKB, T::NT, false, 1, false>;
-  using Epi = GemmEpilogue<OpF16, OUT_F16>;
-  DmaParams p{static_cast<const char *>(a), nullptr, M, N, K * 2, nullptr};
-  typename YL::Params yp{static_cast<const char *>(bt), N, K * 2, K * 2};
-  typename Epi::Params ep{c, M, N};
-  const int nk = K * 2 / T::BKB, gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
-  constexpr int lds = 2 * T::STAGE;
-  auto kern = mma_hybrid_kernel<OpF16, T, YL, Epi>;
-  static thread_local bool allowed = false;
-  if (!allowed) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds);
-    if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "unit_gemm_f16_prepared: hipFuncSetAttribute: %s", hipGetErrorString(e));
-    allowed = true;
-  }
-  GridMap gm{gx, gy, gx < 4 ? gx : 4, 1, gx * gy};
-  set_variant("f16gemmbt_hybrid_x%d_y%d_k%d_w%dx%d%s", T::BX, T::BY, T::BKB, T::WX, T::WY, OUT_F16 ? "_h" : "");
-  hipLaunchKernelGGL(kern, dim3(gm.total), dim3(T::NT), lds, s, p, yp, ep, nk, gm);
-  hipError_t e = hipGetLastError();
-  return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "unit_gemm_f16_prepared: launch: %s", hipGetErrorString(e));
-}
-
 // the same operands through registers (any K that is a multiple of 8; small problems)
 template <class T, bool OUT_F16>
 int run_gemm_f16_bt(const void *a, const void *bt, void *c, int M, int N, int K, hipStream_t s) {
@@ -104,14 +145,12 @@ int run_gemm_f16_bt(const void *a, const void *bt, void *c, int M, int N, int K,
 template <bool OUT_F16>
 int gemm_f16_bt(const void *a, const void *bt, void *c, int M, int N, int K, hipStream_t s) {
   const long tiles_big = (long)ceil_div(M, 256) * ceil_div(N, 256);
-  if (M >= 256 && N >= 128 && K % 64 == 0 && K >= 128) {  // tile choice as in gemm_f16 below
-    const long tiles_half = (long)ceil_div(M, 256) * ceil_div(N, 128);
-    const long rounds_big = ceil_div((int)tiles_big, 256), rounds_half = ceil_div((int)tiles_half, 256);
-    const bool big_ok = N >= 256 && tiles_big >= 128;
-    if (big_ok && rounds_big * 100 <= rounds_half * 55)
-      return run_gemm_f16_bt_dma<Tile<256, 256, 128, 2, 4>, 2, OUT_F16>(a, bt, c, M, N, K, s);
-    if (tiles_half >= 128) return run_gemm_f16_bt_hybrid<Tile<256, 128, 128, 2, 2>, OUT_F16>(a, bt, c, M, N, K, s);
-    if (big_ok) return run_gemm_f16_bt_dma<Tile<256, 256, 128, 2, 4>, 2, OUT_F16>(a, bt, c, M, N, K, s);
+  if (K % 32 == 0 && K >= 64) {  // both operands straight into LDS; tile choice as in gemm_f16 below
+    if (gemm_f16_large_tiles(M, N)) {
+      if (K % 64 == 0) return run_gemm_f16_bt_dma<Tile<256, 256, 128, 2, 4>, 2, OUT_F16>(a, bt, c, M, N, K, s);
+      return run_gemm_f16_bt_dma<Tile<256, 256, 64, 2, 4>, 4, OUT_F16>(a, bt, c, M, N, K, s);
+    }
+    return run_gemm_f16_bt_dma<Tile<128, 128, 64, 2, 2>, 4, OUT_F16>(a, bt, c, M, N, K, s, gemm_f16_direct_splits(M, N, K));
   }
   if (M >= 256 && N >= 256 && tiles_big >= 128) return run_gemm_f16_bt<Tile<256, 256, 128, 2, 4>, OUT_F16>(a, bt, c, M, N, K, s);
   return run_gemm_f16_bt<Tile<128, 128, 64, 2, 2>, OUT_F16>(a, bt, c, M, N, K, s);
@@ -174,7 +213,24 @@ int gemm_f16(const void *a, const void *b, void *c, int M, int N, int K, hipStre
     case 7: if (K % 64 == 0 && K >= 128) return run_gemm_f16_hybrid<Tile<256, 256, 128, 4, 2>, OUT_F16>(a, b, c, M, N, K, s); break;
     case 8: if (K % 64 == 0 && K >= 128) return run_gemm_f16_hybrid<Tile<256, 256, 128, 2, 4>, OUT_F16>(a, b, c, M, N, K, s); break;
     case 9: if (K % 64 == 0 && K >= 128) return run_gemm_f16_hybrid<Tile<256, 128, 128, 2, 2>, OUT_F16>(a, b, c, M, N, K, s); break;
+    case 10: if (K % 64 == 0 && K >= 128 && N % 8 == 0) return run_gemm_f16_dma_tr<Tile<256, 256, 128, 2, 4>, 2, OUT_F16>(a, b, c, M, N, K, s); break;
+    case 11: if (K % 32 == 0 && K >= 128 && N % 8 == 0) return run_gemm_f16_dma_tr<Tile<256, 256, 64, 2, 4>, 4, OUT_F16>(a, b, c, M, N, K, s); break;
+    case 12: if (K % 32 == 0 && K >= 128 && N % 8 == 0) return run_gemm_f16_dma_tr<Tile<256, 128, 64, 2, 2>, 4, OUT_F16>(a, b, c, M, N, K, s); break;
+    case 13: if (K % 32 == 0 && K >= 128 && N % 8 == 0) return run_gemm_f16_dma_tr<Tile<128, 256, 64, 2, 2>, 4, OUT_F16>(a, b, c, M, N, K, s); break;
+    case 15: if (K % 32 == 0 && K >= 128 && N % 8 == 0) return run_gemm_f16_dma_tr<Tile<128, 128, 64, 2, 2>, 4, OUT_F16>(a, b, c, M, N, K, s); break;
+    case 16: if (K % 32 == 0 && K >= 128 && N % 8 == 0) return run_gemm_f16_dma_tr<Tile<128, 128, 64, 2, 2>, 6, OUT_F16>(a, b, c, M, N, K, s); break;
+    case 14: if (K % 32 == 0 && K >= 128 && N % 8 == 0) return run_gemm_f16_dma_tr<Tile<256, 128, 64, 2, 2>, 6, OUT_F16>(a, b, c, M, N, K, s); break;
     default: break;
+  }
+  // K a whole number of 64-byte stages and N of 16-byte chunks: both operands straight into LDS, b read back with the
+  // transposing LDS read.  At 4096^3 116 us against 133 us for the register-transposing pipeline below, 2048^3 26
+  // against 39 us, 1024 x 4096 x 4096 45 against 68 us, same bits.
+  if (K % 32 == 0 && K >= 64 && N % 8 == 0) {
+    if (gemm_f16_large_tiles(M, N)) {
+      if (K % 64 == 0) return run_gemm_f16_dma_tr<Tile<256, 256, 128, 2, 4>, 2, OUT_F16>(a, b, c, M, N, K, s);
+      return run_gemm_f16_dma_tr<Tile<256, 256, 64, 2, 4>, 4, OUT_F16>(a, b, c, M, N, K, s);
+    }
+    return run_gemm_f16_dma_tr<Tile<128, 128, 64, 2, 2>, 4, OUT_F16>(a, b, c, M, N, K, s, gemm_f16_direct_splits(M, N, K));
   }
   // K a whole number of 128-byte stages: a straight into LDS, b through the transposing register loader
   // (measured 130 us against 154 us for the all-register pipeline at 4096^3, same bits).  256 x 256 tiles of eight

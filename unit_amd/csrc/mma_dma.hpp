@@ -25,9 +25,29 @@ struct DmaParams {
   int xrows, yrows;
   int ld;         // bytes per row (both operands)
   const int *ysum;  // WS_Y_GIVEN: sum of each Y row's bytes (the int8 weight sums), computed once per weight
+  int ldy = 0;      // YT: bytes per k row of the (K, yrows) Y operand
 };
 
-template <class Op, class T, int NSTAGE, class Epi, int WS, bool XOR_X>
+typedef short v4s __attribute__((ext_vector_type(4)));
+
+// One wave-level direct load (64 lanes x 16 B -> 1 KiB of LDS at lds_addr) written out as instructions.  The compiler
+// makes every LDS read that follows a direct load it knows of wait for all of them (it cannot tell which LDS bytes
+// a load fills); it spares plain reads whose address it can follow, but not the transposing read, and that wait would
+// undo the ring.  Loads issued this way are invisible to it, so the kernel's own vmcnt waits order them alone.
+__device__ __forceinline__ void direct_load_16(const void *src, u32 lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :
+               : "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(src)
+               : "memory");
+}
+
+// YT (16-bit operands only): Y is given reduction-major, (K, yrows) with yrows contiguous -- the fp16 GEMM's b as the
+// reference has it.  Its tile lands in LDS as it lies in memory, [k][BY / 8 chunks of 8 columns], and the MFMA
+// fragments (8 consecutive k of one column per lane) come out of it with the LDS transposing read
+// (ds_read_b64_tr_b16): within 16 lanes, source lanes 4r .. 4r+3 hand in 16 consecutive columns of k row r and lane
+// i receives column i of the four rows.  Two such reads make one fragment.  The chunk position inside a k row is
+// XORed with 4 * (k % 4), so that the four rows of a read fall into different bank groups (rows are 256 or 512 B).
+template <class Op, class T, int NSTAGE, class Epi, int WS, bool XOR_X, bool YT = false>
 __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Epi::Params ep, int nk, GridMap gm) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   const int t = threadIdx.x;
@@ -41,10 +61,21 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
   static_assert(T::BX % (RPL * NW) == 0 && T::BY % (RPL * NW) == 0, "tile rows split evenly over the waves");
   static_assert(KK % 2 == 0, "fragment double buffering needs an even number of k-steps");
   constexpr int LPS = XL + YL;                   // loads per wave per stage
+  constexpr int CPRY = T::BY / 8, RPLY = 64 / CPRY;  // YT: chunks per k row, k rows per wave-level load
+  static_assert(!YT || (CPRY >= 16 && CPRY <= 64 && (T::BKB / 2) % (RPLY * NW) == 0 && YL == T::BKB / 2 / RPLY / NW &&
+                        WS == WS_NONE && !XOR_X), "transposed-Y tile shape");
 
   int bx, by, split;
   gm.locate(blockIdx.x, bx, by, split);
   const int x0 = bx * T::BX, y0 = by * T::BY;
+  const size_t ystep = YT ? (size_t)(T::BKB / 2) * p.ldy : (size_t)T::BKB;  // Y bytes from one stage to the next
+  if (gm.splits > 1) {  // this workgroup's share of the stages: [first, first + nk)
+    const int per = nk / gm.splits, rem = nk % gm.splits;
+    const int first = split * per + (split < rem ? split : rem);
+    nk = per + (split < rem ? 1 : 0);
+    p.x += (size_t)first * T::BKB;
+    p.y += (size_t)first * ystep;
+  }
 
   // per-lane source offsets: lane -> (row, slot) of its KiB, chunk = slot ^ swizzle(row)
   u32 xoff[XL], yoff[YL];
@@ -58,22 +89,37 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
   }
 #pragma unroll
   for (int i = 0; i < YL; ++i) {
-    const int row = (wave * YL + i) * RPL + lrow;
-    int g = y0 + row;
-    g = g < p.yrows ? g : p.yrows - 1;
-    yoff[i] = (u32)g * (u32)p.ld + ((slot ^ swz<T::BKB>(row)) << 4);
+    if constexpr (YT) {
+      const int krow = (wave * YL + i) * RPLY + lane / CPRY;
+      int c = y0 / 8 + ((lane % CPRY) ^ (4 * (krow & 3)));
+      c = c < p.yrows / 8 ? c : p.yrows / 8 - 1;
+      yoff[i] = (u32)krow * (u32)p.ldy + ((u32)c << 4);
+    } else {
+      const int row = (wave * YL + i) * RPL + lrow;
+      int g = y0 + row;
+      g = g < p.yrows ? g : p.yrows - 1;
+      yoff[i] = (u32)g * (u32)p.ld + ((slot ^ swz<T::BKB>(row)) << 4);
+    }
   }
 
   auto issue = [&](int kt) {
     char *buf = lds + (kt % NSTAGE) * T::STAGE;
-    const char *xs = p.x + (size_t)kt * T::BKB, *ys = p.y + (size_t)kt * T::BKB;
+    const char *xs = p.x + (size_t)kt * T::BKB, *ys = p.y + (size_t)kt * ystep;
 #pragma unroll
-    for (int i = 0; i < XL; ++i)
-      __builtin_amdgcn_global_load_lds((gptr_t)(xs + xoff[i]), (lptr_t)(buf + (wave * XL + i) * 1024), 16, 0, 0);
+    for (int i = 0; i < XL; ++i) {
+      if constexpr (YT)
+        direct_load_16(xs + xoff[i], (u32)(uintptr_t)(lptr_t)(buf + (wave * XL + i) * 1024));
+      else
+        __builtin_amdgcn_global_load_lds((gptr_t)(xs + xoff[i]), (lptr_t)(buf + (wave * XL + i) * 1024), 16, 0, 0);
+    }
 #pragma unroll
-    for (int i = 0; i < YL; ++i)
-      __builtin_amdgcn_global_load_lds((gptr_t)(ys + yoff[i]), (lptr_t)(buf + T::XBYTES + (wave * YL + i) * 1024), 16,
-                                       0, 0);
+    for (int i = 0; i < YL; ++i) {
+      if constexpr (YT)
+        direct_load_16(ys + yoff[i], (u32)(uintptr_t)(lptr_t)(buf + T::XBYTES + (wave * YL + i) * 1024));
+      else
+        __builtin_amdgcn_global_load_lds((gptr_t)(ys + yoff[i]), (lptr_t)(buf + T::XBYTES + (wave * YL + i) * 1024),
+                                         16, 0, 0);
+    }
   };
 
   typename Op::acc_t acc[T::TX][T::TY];
@@ -93,6 +139,18 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
   const int xsw = swz<T::BKB>(xrow), ysw = swz<T::BKB>(yrow);
   const int xbase = xrow * T::BKB, ybase = T::XBYTES + yrow * T::BKB;
 
+  // YT: byte offset, inside the Y tile, of what this lane hands to the transposing reads of fragment j at k-step 0,
+  // read 0: k row 8 * half + (lane % 16) / 4, columns 32 j + 16 * ((lane / 16) % 2) + 4 * (lane % 4) .. + 3
+  int ytr[T::TY];
+  if constexpr (YT) {
+    const int jrow = (lane & 15) >> 2, q = lane & 3, g16 = (lane >> 4) & 1;
+#pragma unroll
+    for (int j = 0; j < T::TY; ++j) {
+      const int c = wy * (T::TY * 4) + j * 4 + 2 * g16 + (q >> 1);
+      ytr[j] = (8 * half + jrow) * (T::BY * 2) + ((c ^ (4 * jrow)) << 4) + (q & 1) * 8;
+    }
+  }
+
   v4i xf[2][T::TX], yf[2][T::TY];
   // fragment i of the step's read list: X0, Y0..Y(TY-1), X1..X(TX-1) -- the first MFMA needs
   // only the first two
@@ -100,8 +158,18 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
     const int cx = ((2 * kk + half) ^ xsw) << 4, cy = ((2 * kk + half) ^ ysw) << 4;
     if (idx == 0)
       xf[s][0] = *reinterpret_cast<const v4i *>(stage + xbase + cx);
-    else if (idx <= T::TY)
-      yf[s][idx - 1] = *reinterpret_cast<const v4i *>(stage + ybase + (idx - 1) * 32 * T::BKB + cy);
+    else if (idx <= T::TY) {
+      if constexpr (YT) {
+        typedef __attribute__((address_space(3))) v4s *trptr_t;
+        typedef short v8s __attribute__((ext_vector_type(8)));
+        const char *src = stage + T::XBYTES + ytr[idx - 1] + kk * 16 * (T::BY * 2);
+        const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((trptr_t)(src));
+        const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((trptr_t)(src + 4 * (T::BY * 2)));
+        yf[s][idx - 1] = __builtin_bit_cast(v4i, (v8s)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      } else {
+        yf[s][idx - 1] = *reinterpret_cast<const v4i *>(stage + ybase + (idx - 1) * 32 * T::BKB + cy);
+      }
+    }
     else
       xf[s][idx - T::TY] = *reinterpret_cast<const v4i *>(stage + xbase + (idx - T::TY) * 32 * T::BKB + cx);
   };
@@ -111,8 +179,13 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
   };
   auto issue_one = [&](int kt, int i) {
     char *buf = lds + (kt % NSTAGE) * T::STAGE;
-    const char *xs = p.x + (size_t)kt * T::BKB, *ys = p.y + (size_t)kt * T::BKB;
-    if (i < XL)
+    const char *xs = p.x + (size_t)kt * T::BKB, *ys = p.y + (size_t)kt * ystep;
+    if constexpr (YT) {
+      if (i < XL)
+        direct_load_16(xs + xoff[i], (u32)(uintptr_t)(lptr_t)(buf + (wave * XL + i) * 1024));
+      else
+        direct_load_16(ys + yoff[i - XL], (u32)(uintptr_t)(lptr_t)(buf + T::XBYTES + (wave * YL + (i - XL)) * 1024));
+    } else if (i < XL)
       __builtin_amdgcn_global_load_lds((gptr_t)(xs + xoff[i]), (lptr_t)(buf + (wave * XL + i) * 1024), 16, 0, 0);
     else
       __builtin_amdgcn_global_load_lds((gptr_t)(ys + yoff[i - XL]),
@@ -205,8 +278,11 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
       wsy[j] = n < p.yrows ? p.ysum[n] : 0;
     }
   }
-  Epi::template store<T>(ep, acc, wsx, wsy, x0 + wx * (T::TX * 32), y0 + wy * (T::TY * 32), lane, wave, lds,
-                         gm.splits > 1);
+  if constexpr (Epi::kSplitPlanes)  // every k-split writes a plane of its own: the last argument is the split
+    Epi::template store<T>(ep, acc, wsx, wsy, x0 + wx * (T::TX * 32), y0 + wy * (T::TY * 32), lane, wave, lds, split);
+  else
+    Epi::template store<T>(ep, acc, wsx, wsy, x0 + wx * (T::TX * 32), y0 + wy * (T::TY * 32), lane, wave, lds,
+                           gm.splits > 1);
 }
 
 }  // namespace unit
