@@ -68,7 +68,7 @@ def test_dense_packed_weights_direct_to_registers(dev, oracle, monkeypatch, M, N
     assert np.array_equal(out.cpu().numpy(), oracle.c_dense(a, wp)), U.last_variant()
 
 
-@pytest.mark.parametrize("M,N,K", [(128, 3072, 768), (50, 260, 1040), (1, 128, 8192)])
+@pytest.mark.parametrize("M,N,K", [(128, 768, 3072), (50, 260, 1040), (1, 128, 8192)])
 def test_dense_k_splits_bit_exact(dev, oracle, M, N, K):
     """Few output tiles: the reduction is shared between workgroups (int32 atomics, exact in any order); the output
     buffer's previous contents must not leak into the sums."""
@@ -370,20 +370,28 @@ def test_full_size_properties(dev):
     assert torch.equal(o32, o1.expand(32, -1, -1, -1, -1))
 
 
-@pytest.mark.parametrize("M,N,K", [(512, 8192, 256), (4096, 4096, 128), (2000, 4100, 384), (64, 128, 128), (300, 4096, 144)])
-def test_dense_on_prepared_weight(dev, oracle, M, N, K):
-    """Weight sums folded once (unit_dense_prepare_weight): shapes with whole 128-byte stages and half a chip of
-    256 x 256 tiles run the direct-to-LDS kernel, ragged M / N included; the others fall back to the plain entry.
-    Bit-exact against a . W^T either way."""
+@pytest.mark.parametrize("M,N,K,kernel", [(512, 8192, 256, "prep_dma_x128_y128"), (4096, 4096, 128, "prep_dma_x256_y256"),
+                                          (2000, 4100, 384, "prep_dma_x256_y256"), (64, 128, 128, "prep_dma_x128_y128"),
+                                          (128, 768, 3072, "prep_dma_x128_y128_k64_w2x2_r4_s12"),
+                                          (300, 4096, 144, "i8denserm"), (4096, 4096, 192, "i8denserm")])
+def test_dense_on_prepared_weight(dev, oracle, M, N, K, kernel):
+    """Weight sums folded once (unit_dense_prepare_weight): both operands go global -> LDS directly, on 256 x 256
+    tiles (whole 128-byte stages) where those fill the chip, else on 128 x 128 tiles (whole 64-byte stages), with
+    k-splits when the tiles are few -- the sums are then added by one split only; ragged M / N included.  The other
+    shapes fall back to the plain entry.  Bit-exact against a . W^T either way."""
     a = rng.uniform_u8((M, K), 70 + M)
     w = rng.uniform_s8((N, K), 71 + N)
     p = U.prepare_dense_weight(_t(w, dev))
     assert np.array_equal(p.wsum.cpu().numpy(), w.astype(np.int64).sum(axis=1))
-    out = U.dense(_t(a, dev), p)
+    out = torch.full((M, N), 777, dtype=torch.int32, device=dev)  # k-splits must not add onto what was there
+    from unit_amd import _lib
+    ta = _t(a, dev)
+    _lib.check(_lib.load().unit_dense_u8s8s32_prepared(ta.data_ptr(), p.w.data_ptr(), p.wsum.data_ptr(), out.data_ptr(), M, N, K,
+                                                       torch.cuda.current_stream().cuda_stream))
     torch.cuda.synchronize()
-    big = K % 128 == 0 and -(-M // 256) * -(-N // 256) >= 128
-    assert ("prep_dma" in U.last_variant()) == big, U.last_variant()
+    assert kernel in U.last_variant(), U.last_variant()
     assert np.array_equal(out.cpu().numpy(), oracle.dense_logical(a, w)), U.last_variant()
+    assert torch.equal(U.dense(ta, p), out)
 
 
 def test_dense_on_prepared_weight_extremes(dev, oracle):

@@ -10,30 +10,6 @@
 namespace unit {
 namespace {
 
-// Which all-direct tile: 256 x 256 (eight waves, one workgroup per CU, the least LDS traffic per MFMA) or 128 x 128
-// (four waves, two workgroups per CU).  Measured time per 1024 of K: a round of large tiles 30 us (24 when under 200
-// CUs are busy), a round of 512 small tiles 21.5 us, 13 us when at most 256 are left (one per CU).
-inline bool gemm_f16_large_tiles(int M, int N) {
-  const long tb = (long)ceil_div(M, 256) * ceil_div(N, 256), t128 = (long)ceil_div(M, 128) * ceil_div(N, 128);
-  const double big = (double)((tb + 255) / 256) * (tb <= 200 ? 24.0 : 30.0);
-  const long rest = t128 % 512;
-  const double small = (double)(t128 / 512) * 21.5 + (rest == 0 ? 0.0 : rest <= 256 ? 13.0 : 21.5);
-  return M >= 256 && N >= 256 && big < small;
-}
-
-// k-splits of the 128 x 128 all-direct tiles (f32 output, added with atomics): up to 128 workgroups, and a split's
-// share of K at least 16 x the tile count (the zero fill and the atomics cost in proportion to the output: 1024^3 on
-// 64 tiles runs 14.5 us whole and 15.6 us in two splits, 512 x 512 x 4096 on 16 tiles 35 us whole and 15 us in 8)
-inline int gemm_f16_direct_splits(int M, int N, int K) {
-  int splits = tuning_override("UNIT_AMD_GEMM_F16_SPLITK");
-  if (splits <= 0) {
-    const long t128 = (long)ceil_div(M, 128) * ceil_div(N, 128);
-    const long share = 16 * t128 > 128 ? 16 * t128 : 128;
-    splits = (int)(128 / t128 < K / share ? 128 / t128 : K / share);
-  }
-  return splits < 1 ? 1 : splits;
-}
-
 // Prepared b: (N, K) rows, K-contiguous like a.  Both operands then go global -> LDS directly
 // (no register round trip, no transposition), through a ring of NSTAGE LDS buffers; K a whole
 // number of stages.
@@ -146,11 +122,11 @@ template <bool OUT_F16>
 int gemm_f16_bt(const void *a, const void *bt, void *c, int M, int N, int K, hipStream_t s) {
   const long tiles_big = (long)ceil_div(M, 256) * ceil_div(N, 256);
   if (K % 32 == 0 && K >= 64) {  // both operands straight into LDS; tile choice as in gemm_f16 below
-    if (gemm_f16_large_tiles(M, N)) {
+    if (direct_gemm_large_tiles(M, N)) {
       if (K % 64 == 0) return run_gemm_f16_bt_dma<Tile<256, 256, 128, 2, 4>, 2, OUT_F16>(a, bt, c, M, N, K, s);
       return run_gemm_f16_bt_dma<Tile<256, 256, 64, 2, 4>, 4, OUT_F16>(a, bt, c, M, N, K, s);
     }
-    return run_gemm_f16_bt_dma<Tile<128, 128, 64, 2, 2>, 4, OUT_F16>(a, bt, c, M, N, K, s, gemm_f16_direct_splits(M, N, K));
+    return run_gemm_f16_bt_dma<Tile<128, 128, 64, 2, 2>, 4, OUT_F16>(a, bt, c, M, N, K, s, direct_gemm_k_splits("UNIT_AMD_GEMM_F16_SPLITK", M, N, 2l * K));
   }
   if (M >= 256 && N >= 256 && tiles_big >= 128) return run_gemm_f16_bt<Tile<256, 256, 128, 2, 4>, OUT_F16>(a, bt, c, M, N, K, s);
   return run_gemm_f16_bt<Tile<128, 128, 64, 2, 2>, OUT_F16>(a, bt, c, M, N, K, s);
@@ -226,11 +202,11 @@ int gemm_f16(const void *a, const void *b, void *c, int M, int N, int K, hipStre
   // transposing LDS read.  At 4096^3 116 us against 133 us for the register-transposing pipeline below, 2048^3 26
   // against 39 us, 1024 x 4096 x 4096 45 against 68 us, same bits.
   if (K % 32 == 0 && K >= 64 && N % 8 == 0) {
-    if (gemm_f16_large_tiles(M, N)) {
+    if (direct_gemm_large_tiles(M, N)) {
       if (K % 64 == 0) return run_gemm_f16_dma_tr<Tile<256, 256, 128, 2, 4>, 2, OUT_F16>(a, b, c, M, N, K, s);
       return run_gemm_f16_dma_tr<Tile<256, 256, 64, 2, 4>, 4, OUT_F16>(a, b, c, M, N, K, s);
     }
-    return run_gemm_f16_dma_tr<Tile<128, 128, 64, 2, 2>, 4, OUT_F16>(a, b, c, M, N, K, s, gemm_f16_direct_splits(M, N, K));
+    return run_gemm_f16_dma_tr<Tile<128, 128, 64, 2, 2>, 4, OUT_F16>(a, b, c, M, N, K, s, direct_gemm_k_splits("UNIT_AMD_GEMM_F16_SPLITK", M, N, 2l * K));
   }
   // K a whole number of 128-byte stages: a straight into LDS, b through the transposing register loader
   // (measured 130 us against 154 us for the all-register pipeline at 4096^3, same bits).  256 x 256 tiles of eight

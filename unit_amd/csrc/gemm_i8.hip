@@ -38,7 +38,8 @@ int run_dense(const void *a, const void *w, void *c, int M, int N, int K, hipStr
 // direct-to-LDS variant: row-major weights, K a whole number of stages.  wsum: the weight's row sums when they
 // were prepared beforehand (unit_dense_prepare_weight), else null and the kernel sums the fragments itself.
 template <class T, int NSTAGE, bool GIVEN = false>
-int run_dense_dma(const void *a, const void *w, void *c, int M, int N, int K, hipStream_t s, const int *wsum = nullptr) {
+int run_dense_dma(const void *a, const void *w, void *c, int M, int N, int K, hipStream_t s, const int *wsum = nullptr,
+                  int splits = 1) {
   using Epi = GemmEpilogue<OpI8, false>;
   DmaParams p{static_cast<const char *>(a), static_cast<const char *>(w), M, N, K, wsum};
   typename Epi::Params ep{c, M, N};
@@ -53,8 +54,14 @@ int run_dense_dma(const void *a, const void *w, void *c, int M, int N, int K, hi
     if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "unit_dense_u8s8s32: hipFuncSetAttribute: %s", hipGetErrorString(e));
     allowed = true;
   }
-  GridMap gm{gx, gy, gx < 4 ? gx : 4, 1, gx * gy};
-  set_variant("i8dense%sdma_x%d_y%d_k%d_w%dx%d_r%d", GIVEN ? "prep_" : "", T::BX, T::BY, T::BKB, T::WX, T::WY, NSTAGE);
+  splits = splits < 1 || (size_t)M * N * 4 % 16 ? 1 : (splits > nk ? nk : splits);
+  if (splits > 1) {  // the k-ranges add into c with atomics (exact for int32)
+    const size_t n16 = (size_t)M * N * 4 / 16;
+    hipLaunchKernelGGL(zero_fill, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, s, static_cast<v4i *>(c), n16);
+  }
+  GridMap gm{gx, gy, gx < 4 ? gx : 4, splits, gx * gy * splits};
+  set_variant("i8dense%sdma_x%d_y%d_k%d_w%dx%d_r%d_s%d", GIVEN ? "prep_" : "", T::BX, T::BY, T::BKB, T::WX, T::WY, NSTAGE,
+              splits);
   hipLaunchKernelGGL(kern, dim3(gm.total), dim3(T::NT), lds, s, p, ep, nk, gm);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "unit_dense_u8s8s32: launch: %s", hipGetErrorString(e));
@@ -121,8 +128,16 @@ int dense(const void *a, const void *w, void *c, int M, int N, int K, unit_strea
     case 13: if (PACKED) return run_dense_mixed(a, w, c, M, N, K, s); break;
     case 14: return run_dense<Tile<256, 256, 128, 2, 4>, PACKED>(a, w, c, M, N, K, s);
     case 15: return run_dense<Tile<256, 256, 128, 4, 2>, PACKED>(a, w, c, M, N, K, s);
+    case 16: if (!PACKED && K % 128 == 0) return run_dense_dma<Tile<256, 256, 128, 4, 2>, 2>(a, w, c, M, N, K, s); break;
+    case 17: if (!PACKED && K % 64 == 0) return run_dense_dma<Tile<128, 128, 64, 2, 2>, 4>(a, w, c, M, N, K, s); break;
     default: break;
   }
+  // row-major weights, K a whole number of 64-byte stages, and a shape that 128 x 128 tiles fill better than 256 x 256
+  // ones: both operands global -> LDS directly, two workgroups per CU (2048^3 23.3 -> 20.7 us, 1024 x 4096 x 4096
+  // 39.8 -> 32.7 us, 8192 x 1024 x 1024 24.6 -> 18.0 us)
+  if (!PACKED && K % 64 == 0 && !direct_gemm_large_tiles(M, N))
+    return run_dense_dma<Tile<128, 128, 64, 2, 2>, 4>(a, w, c, M, N, K, s, nullptr,
+                                                      direct_gemm_k_splits("UNIT_AMD_DENSE_SPLITK", M, N, K));
   if (M >= 256 && N >= 256 && tiles_big >= 128)
     return K % 128 ? run_dense<Tile<256, 256, 128, 2, 4>, PACKED>(a, w, c, M, N, K, s)
                    : run_dense<Tile<256, 256, 128, 2, 4>, PACKED, false>(a, w, c, M, N, K, s);
@@ -165,15 +180,18 @@ extern "C" int unit_dense_u8s8s32_prepared(const void *a, const void *w, const i
   using namespace unit;
   const char *what = "unit_dense_u8s8s32_prepared";
   if (!a || !w || !wsum || !c) return fail(UNIT_E_ARG, "%s: null pointer", what);
-  // the direct-to-LDS kernel needs whole 128-byte stages and pays from half a chip of 256 x 256 tiles on;
+  // the direct-to-LDS kernels need whole stages (128 bytes for the 256 x 256 tiles, 64 for the 128 x 128 ones);
   // everything else runs the plain entry point, which sums the weights itself (same result)
-  const long tiles = (long)ceil_div(M, 256) * ceil_div(N, 256);
-  if (M <= 0 || N <= 0 || K <= 0 || K % 128 || N % 4 || tiles < 128 || row_slice(M, (size_t)K, (size_t)N * 4) ||
+  const bool large = M > 0 && N > 0 && direct_gemm_large_tiles(M, N);
+  if (M <= 0 || N <= 0 || K <= 0 || K % (large ? 128 : 64) || N % 4 || row_slice(M, (size_t)K, (size_t)N * 4) ||
       !fits((size_t)M * K) || !fits((size_t)N * K) || !fits((size_t)M * N * 4))
     return unit_dense_u8s8s32(a, w, c, M, N, K, stream);
   if (int rc = check_aligned(what, {a, w, c})) return rc;
   if (int rc = check_device()) return rc;
-  return run_dense_dma<Tile<256, 256, 128, 4, 2>, 2, true>(a, w, c, M, N, K, static_cast<hipStream_t>(stream), wsum);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (large) return run_dense_dma<Tile<256, 256, 128, 4, 2>, 2, true>(a, w, c, M, N, K, s, wsum);
+  return run_dense_dma<Tile<128, 128, 64, 2, 2>, 4, true>(a, w, c, M, N, K, s, wsum,
+                                                          direct_gemm_k_splits("UNIT_AMD_DENSE_SPLITK", M, N, K));
 }
 
 extern "C" int unit_dense_dotprod_u8s8s32(const void *a, const void *wp, void *c, int32_t M, int32_t N, int32_t K,

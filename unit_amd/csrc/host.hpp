@@ -123,6 +123,32 @@ inline int gemm_k_splits(const char *env, int M, int N, long kbytes, int nk) {
   return splits < 1 ? 1 : (splits > nk ? nk : splits);
 }
 
+// Which all-direct GEMM tile (both operands global -> LDS): 256 x 256 (eight waves, one workgroup per CU, the least LDS
+// traffic per MFMA) or 128 x 128 (four waves, two workgroups per CU).  Measured time per 2048 reduction bytes (fp16):
+// a round of large tiles 30 us (24 when under 200 CUs are busy), a round of 512 small tiles 21.5 us, 13 us when at
+// most 256 are left (one per CU).
+inline bool direct_gemm_large_tiles(int M, int N) {
+  const long tb = (long)ceil_div(M, 256) * ceil_div(N, 256), t128 = (long)ceil_div(M, 128) * ceil_div(N, 128);
+  const double big = (double)((tb + 255) / 256) * (tb <= 200 ? 24.0 : 30.0);
+  const long rest = t128 % 512;
+  const double small = (double)(t128 / 512) * 21.5 + (rest == 0 ? 0.0 : rest <= 256 ? 13.0 : 21.5);
+  return M >= 256 && N >= 256 && big < small;
+}
+
+// k-splits of the 128 x 128 all-direct tiles (results added with atomics into the zero-filled output): up to 128
+// workgroups, and a split's share of the reduction at least 32 bytes x the tile count (the zero fill and the atomics
+// cost in proportion to the output: fp16 1024^3 on 64 tiles runs 14.5 us whole and 15.6 us in two splits,
+// 512 x 512 x 4096 on 16 tiles 35 us whole and 15 us in 8).  The environment variable pins the count.
+inline int direct_gemm_k_splits(const char *env, int M, int N, long kbytes) {
+  int splits = tuning_override(env);
+  if (splits <= 0) {
+    const long t128 = (long)ceil_div(M, 128) * ceil_div(N, 128);
+    const long share = 32 * t128 > 256 ? 32 * t128 : 256;
+    splits = (int)(128 / t128 < kbytes / share ? 128 / t128 : kbytes / share);
+  }
+  return splits < 1 ? 1 : splits;
+}
+
 // Enqueue mma_kernel over gx x gy tiles and `splits` k-ranges.  With splits > 1 the epilogue
 // accumulates with atomics, so `out` (out_bytes, a multiple of 16) is zero-filled first.
 template <class Op, class T, class XL, class YL, class Epi, int WS>

@@ -215,13 +215,18 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
         if (j == T::TY - 1 && i + 1 < T::TX) xf[s][i + 1] ^= (int)0x80808080;
       }
       if constexpr (WS == WS_Y) {
-        // TY fragments x 4 dwords spread over the first 4*TY MFMAs
-        if (m < 4 * T::TY) wsy[m / 4] = __builtin_amdgcn_sdot4(yf[s][m / 4][m % 4], 0x01010101, wsy[m / 4], false);
+        // TY fragments x 4 dwords spread over the step's MFMAs, DPM dots after each
+        constexpr int DPM = (4 * T::TY + NM - 1) / NM;
+#pragma unroll
+        for (int d = 0; d < DPM; ++d) {
+          const int w = m * DPM + d;
+          if (w < 4 * T::TY) wsy[w / 4] = __builtin_amdgcn_sdot4(yf[s][w / 4][w % 4], 0x01010101, wsy[w / 4], false);
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
     }
   };
-  static_assert(T::TX * T::TY >= LPS && T::TX * T::TY >= T::TX + T::TY && (WS != WS_Y || T::TX * T::TY >= 4 * T::TY),
+  static_assert(T::TX * T::TY >= LPS && T::TX * T::TY >= T::TX + T::TY,
                 "not enough MFMAs per k-step to carry the step's other work");
 
   // One stage.  ISSUE: stage kt + NSTAGE exists and is fetched into the buffer this stage
@@ -275,7 +280,7 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
 #pragma unroll
     for (int j = 0; j < T::TY; ++j) {
       const int n = y0 + wy * (T::TY * 32) + j * 32 + l32;
-      wsy[j] = n < p.yrows ? p.ysum[n] : 0;
+      wsy[j] = n < p.yrows && split == 0 ? p.ysum[n] : 0;  // one k-split adds the whole row's sum
     }
   }
   if constexpr (Epi::kSplitPlanes)  // every k-split writes a plane of its own: the last argument is the split
