@@ -258,16 +258,23 @@ __global__ __launch_bounds__(256) void add_planes(const v4f *__restrict__ ws, vo
 int gemm_f16_planes(const char *what, const void *a, const void *b, void *c, int M, int N, int K, bool out_f16, void *ws,
                     int splits, hipStream_t s) {
   using T = SplitTile;
-  using XL = RowMajorLoader<T::BX, T::BKB, T::NT, false, 1, true>;
-  using YL = KMajorF16Loader<T::BY, T::BKB, T::NT, 1, true>;
-  typename XL::Params xp{static_cast<const char *>(a), M, K * 2, K * 2};
-  typename YL::Params yp{static_cast<const char *>(b), N, K, N + 4, 0, N * 2};
   const size_t plane = (size_t)M * N * 4;
   GemmPlaneEpilogue::Params ep{ws, M, N, plane};
-  const int nk = ceil_div(K * 2, T::BKB), gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
-  set_variant("f16gemm_planes_x%d_y%d_k%d_w%dx%d%s_s%d", T::BX, T::BY, T::BKB, T::WX, T::WY, out_f16 ? "_h" : "", splits);
-  if (int rc = launch_mma<OpF16, T, XL, YL, GemmPlaneEpilogue, WS_NONE>(xp, yp, ep, nk, gx, gy, 4, splits, nullptr, 0, 0, s, what))
-    return rc;
+  if (K % 32 == 0 && N % 8 == 0 && splits <= K * 2 / T::BKB) {
+    // whole 64-byte stages: both operands global -> LDS directly, b read back with the transposing LDS read
+    if (int rc = run_gemm_f16_dma_tr<T, 4, GemmPlaneEpilogue>(what, out_f16 ? "planes_dmatr_h" : "planes_dmatr", a, b, ep, M, N,
+                                                              K, splits, nullptr, s))
+      return rc;
+  } else {
+    using XL = RowMajorLoader<T::BX, T::BKB, T::NT, false, 1, true>;
+    using YL = KMajorF16Loader<T::BY, T::BKB, T::NT, 1, true>;
+    typename XL::Params xp{static_cast<const char *>(a), M, K * 2, K * 2};
+    typename YL::Params yp{static_cast<const char *>(b), N, K, N + 4, 0, N * 2};
+    const int nk = ceil_div(K * 2, T::BKB), gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
+    set_variant("f16gemm_planes_x%d_y%d_k%d_w%dx%d%s_s%d", T::BX, T::BY, T::BKB, T::WX, T::WY, out_f16 ? "_h" : "", splits);
+    if (int rc = launch_mma<OpF16, T, XL, YL, GemmPlaneEpilogue, WS_NONE>(xp, yp, ep, nk, gx, gy, 4, splits, nullptr, 0, 0, s, what))
+      return rc;
+  }
   const size_t n4 = (size_t)M * N / 4;
   if (out_f16)
     hipLaunchKernelGGL(add_planes<true>, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s, static_cast<const v4f *>(ws), c,
