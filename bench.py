@@ -76,7 +76,7 @@ def main():
     ap.add_argument("--profile", default=None, metavar="WHAT",
                     help="launch one kernel 20 times and exit (for rocprofv3): a ResNet-50 layer name such as "
                          "3x3_256_256@14 (append :f16 for the fp16 convolution, :cold to cycle operand copies), "
-                         "or gemm_i8 / gemm_f16 / gemm_f16_prepared / copy / pack_u8")
+                         "or gemm_i8 / gemm_i8_prepared / gemm_f16 / gemm_f16_prepared / gemm_f16_2048 / copy / pack_u8")
     ap.add_argument("--profile-batch", type=int, default=None, metavar="N",
                     help="batch of the --profile launches of a layer (default: the benchmark's 32)")
     args = ap.parse_args()
@@ -126,13 +126,17 @@ def main():
         return sorted(seen)[len(seen) // 2] if median else min(seen)
 
     prof, prof_mode = (args.profile.split(":") + [""])[:2] if args.profile else (None, "")
-    if prof in ("gemm_i8", "gemm_f16", "gemm_f16_prepared", "copy", "pack_u8"):
-        n = 4096
+    if prof in ("gemm_i8", "gemm_i8_prepared", "gemm_f16", "gemm_f16_prepared", "gemm_f16_2048", "copy", "pack_u8"):
+        n = 2048 if prof.endswith("_2048") else 4096
         if prof == "gemm_i8":
             a = dev_t(rng.uniform_u8((n, n), 11))
             w = dev_t(rng.uniform_s8((n, n), 12))
             fn = lambda: U.dense(a, w)
-        elif prof == "gemm_f16":
+        elif prof == "gemm_i8_prepared":
+            a = dev_t(rng.uniform_u8((n, n), 11))
+            pw = U.prepare_dense_weight(dev_t(rng.uniform_s8((n, n), 12)))
+            fn = lambda: U.dense(a, pw)
+        elif prof in ("gemm_f16", "gemm_f16_2048"):
             a = dev_t(rng.normal_f16((n, n), 13, 1.0 / 64))
             b = dev_t(rng.normal_f16((n, n), 14))
             fn = lambda: U.gemm_fp16(a, b)
