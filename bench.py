@@ -283,7 +283,9 @@ def main():
         try:
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
+                stream = torch.cuda.current_stream().cuda_stream  # the launches go to the capturing stream
                 step()
+            stream = torch.cuda.current_stream().cuda_stream
             graph_ms, graph_wall_ms = timed(graph.replay)
             # replays must reproduce the eager outputs bit for bit
             keep = [ly["out"].clone() for ly in layers]
