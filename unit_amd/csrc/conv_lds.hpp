@@ -9,10 +9,12 @@
 // row consecutive in memory.  One direct load moves (64 pixel rows) x (one tap): lane i fetches the 16
 // bytes of row i -- coalesced along the image row -- and they land in LDS as [tap slot][row][16 bytes],
 // which is also the conflict-free order for the fragment reads (lanes 0-31 one tap, 32-63 the next, 32
-// consecutive rows each).  Zero padding is address selection: a lane whose tap falls outside the image
-// fetches a 16-byte line of zeros instead (kept behind the prepared weights), so there are no masks on
-// the data path; the u8 -> s8 shift is one XOR per fragment dword after the fragment read, its
-// correction 128 * sum(w) comes precomputed with the prepared weights.
+// consecutive rows each).  Zero padding is the hardware's: the pixel loads are raw buffer loads over the data
+// tensor, a lane whose tap falls outside the image is given an offset past the tensor, and an out-of-range lane
+// of a buffer load stores zeros -- no masks or selects on the data path.  The lane's offset of each window
+// position is computed once per workgroup into an LDS table; per load the wave reads one entry and adds the
+// channel block's offset as the load's scalar offset.  The u8 -> s8 shift is one XOR per fragment dword after
+// the fragment read, its correction 128 * sum(w) comes precomputed with the prepared weights.
 //
 // Pipeline.  Stage kt (KS k-steps) is computed from buffer kt % NST while the direct loads of stage
 // kt + NST - 1 are issued into the buffer that stage kt - 1 freed, spread over the stage's MFMAs, and the
@@ -53,6 +55,20 @@ struct LdsShape {
   static_assert(NT <= 1024 && NST >= 3 && NST <= 6, "at most 16 waves; ring of 3 to 6 buffers");
 };
 
+// The direct loads are written out as instructions, so that the compiler's counter bookkeeping does not see
+// them (it would make LDS reads that follow a direct load wait for all of them); the kernel's own vmcnt waits
+// order them.  Weight fragments: scalar base + the lane's 16-byte offset.  Pixel rows: a raw buffer load, whose
+// out-of-range lanes store zeros into LDS -- the hardware's own zero padding.
+__device__ __forceinline__ void dma_global_16(u32 lds_addr, u32 voff, const void *sbase) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+}
+__device__ __forceinline__ void dma_buffer_16(u32 lds_addr, u32 voff, v4i rsrc, u32 soff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
+               : "memory");
+}
+
 template <class S, bool SHIFT, bool Q8 = false, bool NCHW = false>
 __global__ __launch_bounds__(S::NT) void conv_lds(const char *__restrict__ data, const char *__restrict__ wgt,
                                                   const char *__restrict__ zero, typename ConvEpilogue<OpI8>::Params ep,
@@ -60,46 +76,36 @@ __global__ __launch_bounds__(S::NT) void conv_lds(const char *__restrict__ data,
   using Op = OpI8;
   extern __shared__ __attribute__((aligned(16))) char lds[];
   constexpr int TX = S::TX, TY = S::TY, KG = S::KG, KS = S::KS, NST = S::NST, LW = S::LW, NM = S::NM, NF = S::NF;
-  constexpr int LPK = S::LPK, LY = S::LY;
+  constexpr int LPK = S::LPK, LX = S::LX, LY = S::LY;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int grp = wave / S::NWG, wg = wave % S::NWG;
   const int wx = wg % S::WX, wy = wg / S::WX;
   const int l32 = lane & 31, half = lane >> 5;
 
-  // k-steps [s0, s1) of this k-group, in stages of KS; every group runs `rounds` stages (one barrier each),
-  // a group with fewer k-steps computes nothing in the surplus ones
+  // k-steps [s0, s1) of this k-group, in stages of KS; every group runs `rounds` stages (one barrier each).  The
+  // k-steps of a last stage that lie past s1 are computed on zero weights.
   const int s0 = nsteps * grp / KG, s1 = nsteps * (grp + 1) / KG;
   const int rounds = ((nsteps + KG - 1) / KG + KS - 1) / KS;
   const int nst = (s1 - s0 + KS - 1) / KS;
-
-  // tap (ci, kh, kw) -> (byte offset of the tap relative to the window origin, window position kh * KW + kw);
-  // entries past the last tap point at position 31, which no pixel has inside: they fetch zeros
-  v2i *tab = reinterpret_cast<v2i *>(lds + S::kMain);
-  const int ntab = 2 * (nsteps + KG * KS);
-  for (int e = threadIdx.x; e < ntab; e += S::NT) {
-    v2i ent = {0, 31};
-    if (e < g.ntaps) {
-      int kw, rest, kh, ci;
-      g.by_kw.divmod(e, rest, kw);
-      g.by_kh.divmod(rest, ci, kh);
-      ent[0] = ((ci * g.H + kh * g.dh) * g.W + kw * g.dw) * 16;
-      ent[1] = kh * g.KW + kw;
-    }
-    tab[e] = ent;
-  }
 
   int bx, by, split;
   gm.locate(blockIdx.x, bx, by, split);
   const int x0 = bx * S::BX, y0 = by * S::BY;
   char *ring = lds + grp * S::RING;
+  const u32 ring_addr = (u32)(uintptr_t)(lptr_t)ring;
 
-  // pixel side: this wave gathers rows rg * 64 + lane of the tile
-  const int rg = wg % S::RG;
-  u32 inside = 0;  // window positions (kh, kw) inside the image; none for rows past the last pixel
-  int pixoff = 0;  // byte offset of the window origin (may lie before the tensor at the borders)
-  {
-    const int m = y0 + rg * 64 + lane;
+  // Position table, per 64-row group of the tile: postab[rg][p][lane] = byte offset in the data tensor of window
+  // position p = kh * KW + kw of the row's pixel, channel block 0 -- or an offset past the tensor when that position
+  // lies outside the image (or the row is past the last pixel): the buffer load then stores zeros.  Row npos is
+  // out of range for every lane (taps past the last one).
+  const int npos = g.KH * g.KW;
+  constexpr u32 kOutside = 0x80000000u;
+  u32 *postab = reinterpret_cast<u32 *>(lds + S::kMain);
+  if (wave < S::RG) {
+    const int m = y0 + wave * 64 + lane;
+    u32 inside = 0;
+    int pixoff = 0;
     if (m < g.npix) {
       int n, rem, oh, ow;
       g.by_ohw.divmod(m, n, rem);
@@ -112,12 +118,54 @@ __global__ __launch_bounds__(S::NT) void conv_lds(const char *__restrict__ data,
         if ((u32)(ih0 + kh * g.dh) < (u32)g.H) bits |= cols << (kh * g.KW);
       inside = bits;
     }
+    u32 *mine = postab + wave * (npos + 1) * 64 + lane;
+    int p = 0;
+    for (int kh = 0; kh < g.KH; ++kh)
+      for (int kw = 0; kw < g.KW; ++kw, ++p)
+        mine[p * 64] = ((inside >> p) & 1u) ? (u32)(pixoff + (kh * g.dh * g.W + kw * g.dw) * 16) : kOutside;
+    mine[npos * 64] = kOutside;
   }
+
   const int lastkb = (ep.K - 1) >> 5;
   const u32 lane16 = (u32)lane * 16u;
-  // one of 256 lines of zeros, by workgroup and wave, so that the padded taps of the whole grid do not all queue
-  // at one L2 channel
-  const char *zline = zero + (((u32)blockIdx.x * 5u + (u32)wave * 3u) & 255u) * 64u;
+  // raw buffer over the data tensor (base, no stride, size in bytes)
+  v4i rsrc;
+  {
+    const unsigned long long base = (unsigned long long)data;
+    rsrc[0] = __builtin_amdgcn_readfirstlane((int)(u32)base);
+    rsrc[1] = __builtin_amdgcn_readfirstlane((int)((u32)(base >> 32) & 0xffffu));
+    rsrc[2] = __builtin_amdgcn_readfirstlane((int)((u32)g.N * g.img_bytes));
+    rsrc[3] = 0x00020000;
+  }
+
+  // ---- this wave's direct loads of a stage, as scalar state that advances from stage to stage (they are issued
+  // strictly in stage order): LX weight fragments (KiB q = wg + n * NWG of the stage's X part: k-step q / XB,
+  // channel block q % XB), then LY pixel loads (KiB q of the Y part: tap slot q / RG of the stage, row group q % RG)
+  const char *xsrc[LX];
+  int xs[LX];
+#pragma unroll
+  for (int n = 0; n < LX; ++n) {
+    const int q = wg + n * S::NWG, ks = q / S::XB, xb = q % S::XB;
+    int kb = (x0 >> 5) + xb;
+    kb = kb < lastkb ? kb : lastkb;
+    xs[n] = s0 + ks;
+    xsrc[n] = wgt + ((size_t)kb * nsteps + xs[n]) * 1024;
+  }
+  const int rg = wg % S::RG;
+  const u32 chw16 = (u32)g.H * (u32)g.W * 16u;  // bytes from one 16-channel block of an image to the next
+  const int step_ci = g.by_kh.div(g.by_kw.div(2 * KS)), step_pos = 2 * KS - step_ci * npos;  // taps per stage = ci blocks + positions
+  int ytap[LY], ypos[LY];
+  u32 yci[LY];
+#pragma unroll
+  for (int n = 0; n < LY; ++n) {
+    const int t = 2 * s0 + (wg + n * S::NWG) / S::RG;
+    const int ci = g.by_kh.div(g.by_kw.div(t));
+    ytap[n] = t;
+    ypos[n] = t - ci * npos;
+    yci[n] = (u32)ci * chw16;
+  }
+  const u32 *posrow = postab + rg * (npos + 1) * 64 + lane;
+  u32 yvoff[LY];  // the lane's offsets of the pixel loads about to be issued, read from the position table
 
   // per-channel addends of the blocks this wave writes back, fetched now so that the latency hides behind the loop
   int addv[S::NBW];
@@ -133,34 +181,34 @@ __global__ __launch_bounds__(S::NT) void conv_lds(const char *__restrict__ data,
       }
     }
   }
-  __syncthreads();  // tap table visible
+  __syncthreads();  // position table visible
 
-  // the tap table entries of this wave's pixel loads for one stage, read ahead of their use
-  v2i ent[LY];
-  auto read_taps = [&](int st) {
-    const int sb = s0 + st * KS;
-#pragma unroll
-    for (int n = 0; n < LY; ++n) ent[n] = tab[2 * sb + (wg + n * S::NWG) / S::RG];
+  int iss_off = 0;  // ring buffer (byte offset) of the stage whose loads are being issued
+  auto bump = [](int off) { return off + S::STAGE == S::RING ? 0 : off + S::STAGE; };
+  // offset of pixel load n (LX .. LW-1) out of the position table, to be read some MFMAs before the load is issued
+  auto read_voff = [&](int n) {
+    const int k = n - LX;
+    const int row = ytap[k] < g.ntaps ? ypos[k] : npos;
+    yvoff[k] = posrow[row * 64];
   };
-  // direct load n (0 .. LW-1) of this wave for stage st: first its share of the weight fragments, then of the
-  // pixel rows (tap table entries in `ent`)
-  auto issue_one = [&](int st, int n) {
-    const int sb = s0 + st * KS;
-    char *slot = ring + (st % NST) * S::STAGE;
-    if (n < S::LX) {
-      const int q = wg + n * S::NWG, ks = q / S::XB, xb = q % S::XB;
-      int kb = (x0 >> 5) + xb;
-      kb = kb < lastkb ? kb : lastkb;
-      int s = sb + ks;
-      s = s < nsteps - 1 ? s : nsteps - 1;  // surplus k-steps of a last stage re-read the last one; they are not computed
-      const char *src = wgt + ((size_t)kb * nsteps + s) * 1024;
-      __builtin_amdgcn_global_load_lds((gptr_t)(src + lane16), (lptr_t)(slot + q * 1024), 16, 0, 0);
+  // direct load n (0 .. LW-1) of the stage being issued; advances the load's state to the next stage
+  auto issue_one = [&](int n) {
+    if (n < LX) {
+      const int q = wg + n * S::NWG;
+      const char *src = xs[n] < s1 ? xsrc[n] : zero;
+      dma_global_16(ring_addr + iss_off + q * 1024, lane16, src);
+      xs[n] += KS;
+      xsrc[n] += KS * 1024;
     } else {
-      const int q = wg + (n - S::LX) * S::NWG;
-      const v2i e = ent[n - S::LX];
-      const char *src = data + (u32)(pixoff + e[0]);
-      src = ((inside >> e[1]) & 1u) ? src : zline;
-      __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(slot + S::XPART + q * 1024), 16, 0, 0);
+      const int k = n - LX, q = wg + k * S::NWG;
+      dma_buffer_16(ring_addr + iss_off + S::XPART + q * 1024, yvoff[k], rsrc, yci[k]);
+      ytap[k] += 2 * KS;
+      ypos[k] += step_pos;
+      yci[k] += (u32)step_ci * chw16;
+      if (ypos[k] >= npos) {
+        ypos[k] -= npos;
+        yci[k] += chw16;
+      }
     }
   };
 
@@ -184,21 +232,25 @@ __global__ __launch_bounds__(S::NT) void conv_lds(const char *__restrict__ data,
       xf[s][i] = *reinterpret_cast<const v4i *>(slot + xfrag + (ks * S::XB + i) * 1024);
   };
   // One k-step: every MFMA is followed by one slice of the stage's other work (a fragment read for the next
-  // k-step, a direct load for stage issue_st, the shift of the next pixel fragment) and a scheduling fence.
-  //   s: fragment slot consumed; rd_slot / rd_ks: where the next k-step's fragments come from (has_read);
-  //   dl0: index of the first direct load this k-step issues, LPK of them (has_issue); live: the k-step counts
-  auto step = [&](int s, const char *rd_slot, int rd_ks, int issue_st, int dl0, auto has_read, auto has_issue,
-                  auto live) {
+  // k-step, the table read or the issue of a direct load, the shift of the next pixel fragment) and a scheduling
+  // fence.  s: fragment slot consumed; rd_slot / rd_ks: where the next k-step's fragments come from (has_read);
+  // dl0: index of the first direct load this k-step issues, LPK of them (has_issue).
+  auto step = [&](int s, const char *rd_slot, int rd_ks, int dl0, auto has_read, auto has_issue) {
     if constexpr (SHIFT) yf[s][0] ^= (int)0x80808080;
 #pragma unroll
     for (int m = 0; m < NM; ++m) {
       const int i = m / TY, j = m % TY;
-      if constexpr (decltype(live)::value) acc[i][j] = Op::mma(xf[s][i], yf[s][j], acc[i][j]);
+      acc[i][j] = Op::mma(xf[s][i], yf[s][j], acc[i][j]);
       if constexpr (decltype(has_read)::value) {
         if (m < NF) load_one(rd_slot, rd_ks, s ^ 1, m);
       }
       if constexpr (decltype(has_issue)::value) {
-        if (m >= NM - LPK && dl0 + (m - (NM - LPK)) < LW) issue_one(issue_st, dl0 + (m - (NM - LPK)));
+        if (m == 0) {
+#pragma unroll
+          for (int d = 0; d < LPK; ++d)
+            if (dl0 + d >= LX && dl0 + d < LW) read_voff(dl0 + d);
+        }
+        if (m >= NM - LPK && dl0 + (m - (NM - LPK)) < LW) issue_one(dl0 + (m - (NM - LPK)));
       }
       if constexpr (SHIFT) {
         if (m + 1 < TY) yf[s][m + 1] ^= (int)0x80808080;
@@ -209,21 +261,17 @@ __global__ __launch_bounds__(S::NT) void conv_lds(const char *__restrict__ data,
   using yes = std::integral_constant<bool, true>;
   using no = std::integral_constant<bool, false>;
 
-  // Stage st.  AHEAD: stage st + NST - 1 exists and is fetched during this stage; NEXT: stage st + 1 exists.
-  // The k-steps of the group's last stage that lie past s1 are skipped (the branch is uniform).
-  auto stage = [&](int st, auto ahead, auto next) {
-    const char *cur = ring + (st % NST) * S::STAGE;
-    const char *nxt = ring + ((st + 1) % NST) * S::STAGE;
-    const int sb = s0 + st * KS;
-    if constexpr (decltype(ahead)::value) read_taps(st + NST - 1);
+  // Stage st, computed from ring buffer cur_off.  AHEAD: stage st + NST - 1 exists and is fetched during this stage
+  // (into iss_off); NEXT: stage st + 1 exists.
+  int st = 0, cur_off = 0;
+  auto stage = [&](auto ahead, auto next) {
+    const char *cur = ring + cur_off;
+    const int nxt_off = bump(cur_off);
+    const char *nxt = ring + nxt_off;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const bool on = sb + ks < s1;
       if (ks + 1 < KS) {
-        if (on)
-          step(ks & 1, cur, ks + 1, st + NST - 1, ks * LPK, yes{}, ahead, yes{});
-        else
-          step(ks & 1, cur, ks + 1, st + NST - 1, ks * LPK, yes{}, ahead, no{});
+        step(ks & 1, cur, ks + 1, ks * LPK, yes{}, ahead);
       } else {
         // stage st + 1 must have landed; the stages behind it and the loads of stage st + NST - 1 issued so far may
         // stay in flight.  Towards the end fewer stages are behind: `behind` counts the whole ones.
@@ -245,21 +293,23 @@ __global__ __launch_bounds__(S::NT) void conv_lds(const char *__restrict__ data,
         __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's reads of `cur` are done
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        if (on)
-          step(ks & 1, nxt, 0, st + NST - 1, ks * LPK, next, ahead, yes{});
-        else
-          step(ks & 1, nxt, 0, st + NST - 1, ks * LPK, next, ahead, no{});
+        step(ks & 1, nxt, 0, ks * LPK, next, ahead);
       }
     }
+    if constexpr (decltype(ahead)::value) iss_off = bump(iss_off);
+    cur_off = nxt_off;
+    ++st;
   };
 
   // prologue: stages 0 .. NST - 2 by direct loads, the first fragments
 #pragma unroll
   for (int p = 0; p < NST - 1; ++p)
     if (p < nst) {
-      read_taps(p);
 #pragma unroll
-      for (int n = 0; n < LW; ++n) issue_one(p, n);
+      for (int n = LX; n < LW; ++n) read_voff(n);
+#pragma unroll
+      for (int n = 0; n < LW; ++n) issue_one(n);
+      iss_off = bump(iss_off);
     }
   if (nst >= NST - 1) {
     UNIT_WAIT_VMCNT((NST - 2) * LW);
@@ -270,10 +320,9 @@ __global__ __launch_bounds__(S::NT) void conv_lds(const char *__restrict__ data,
 #pragma unroll
   for (int i = 0; i < NF; ++i) load_one(ring, 0, 0, i);
 
-  int st = 0;
-  for (; st + NST - 1 < nst; ++st) stage(st, yes{}, yes{});
-  for (; st + 1 < nst; ++st) stage(st, no{}, yes{});
-  for (; st < nst; ++st) stage(st, no{}, no{});
+  while (st + NST - 1 < nst) stage(yes{}, yes{});
+  while (st + 1 < nst) stage(no{}, yes{});
+  while (st < nst) stage(no{}, no{});
   // k-groups with fewer stages keep the others company at the barriers
   for (; st < rounds; ++st) __builtin_amdgcn_s_barrier();
 

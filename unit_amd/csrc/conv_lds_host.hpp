@@ -12,7 +12,7 @@ int run_lds(const char *what, const char *tag, const unit_conv_desc *d, const Co
             const int *bias2 = nullptr, int shift = 0, int planar = 0) {
   static_assert(S::kMain + 4096 <= kMaxLds, "variant does not fit the LDS");
   const PreparedLayout pl = prepared_layout(d->K, d->C, d->KH, d->KW, 16, 1);
-  const int lds = S::kMain + 2 * (pl.nsteps + S::KG * S::KS) * 8;  // rings (or write-back areas) + tap table
+  const int lds = S::kMain + S::RG * (d->KH * d->KW + 1) * 256;  // rings (or write-back areas) + position table
   if (lds > kMaxLds) return fail(UNIT_E_ARG, "%s: needs %d bytes of LDS (limit %d)", what, lds, kMaxLds);
   auto kern = conv_lds<S, SHIFT, Q8, NCHW>;
   static thread_local bool allowed = false;  // the opt-in for > 64 KiB of dynamic LDS is sticky per kernel

@@ -9,8 +9,8 @@
 //     fp16: channel kb * 32 + lane % 32, tap s, input channels 8 (lane / 32) .. + 8;
 //   channels past K and the tap that pads an odd tap count are zeros;
 //   int8 only, behind the fragments: int32 addend[kb * 32 + c] = 128 * sum of the channel's weights
-//   (what a u8 convolution computed on x ^ 0x80 has to add back), then 16 KiB of zeros: the lines that the
-//   LDS-shared kernels (conv_lds.hpp) fetch in place of a tap that falls into the zero padding.
+//   (what a u8 convolution computed on x ^ 0x80 has to add back), then 16 KiB of zeros: the weight fragments
+//   that the LDS-shared kernels (conv_lds.hpp) read for k-steps past a k-group's share of the reduction.
 #pragma once
 #include <cstddef>
 
@@ -19,11 +19,10 @@ namespace unit {
 struct PreparedLayout {
   int kblocks, nsteps;
   size_t frag_bytes;    // kblocks * nsteps * 1 KiB
-  size_t total_bytes;   // + the addends and the zero line for int8
-  size_t zero_off;      // int8: byte offset of the zero line
+  size_t total_bytes;   // + the addends and the zero region for int8
+  size_t zero_off;      // int8: byte offset of the zero region
 };
-// 16 KiB of zeros, not one line: every padded tap of every workgroup on the chip fetches from here, and a single
-// line would make one L2 channel the hot spot of the whole kernel; lanes pick a line by workgroup, wave and tap
+// size of the zero region (a wave-level load reads 1 KiB of it; the size is part of the prepared buffer's layout)
 constexpr int kZeroLine = 16384;
 
 inline PreparedLayout prepared_layout(int K, int C, int KH, int KW, int cb, int elem_bytes) {
