@@ -30,10 +30,11 @@ struct DmaParams {
 
 typedef short v4s __attribute__((ext_vector_type(4)));
 
-// One wave-level direct load (64 lanes x 16 B -> 1 KiB of LDS at lds_addr) written out as instructions.  The compiler
-// makes every LDS read that follows a direct load it knows of wait for all of them (it cannot tell which LDS bytes
-// a load fills); it spares plain reads whose address it can follow, but not the transposing read, and that wait would
-// undo the ring.  Loads issued this way are invisible to it, so the kernel's own vmcnt waits order them alone.
+// One wave-level direct load (64 lanes x 16 B -> 1 KiB of LDS at lds_addr) written out as instructions.  A direct
+// load that the compiler knows of costs twice: it counts the load on the LDS counter as well, after which every wait
+// for a fragment read becomes a wait for all of them (lgkmcnt(0) at the head of every k-step), and it makes the
+// transposing LDS read wait for all direct loads in flight (it cannot tell which LDS bytes a load fills), which
+// undoes the ring.  Loads issued this way are invisible to it, so the kernel's own vmcnt waits order them alone.
 __device__ __forceinline__ void direct_load_16(const void *src, u32 lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
                :
@@ -106,20 +107,10 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
     char *buf = lds + (kt % NSTAGE) * T::STAGE;
     const char *xs = p.x + (size_t)kt * T::BKB, *ys = p.y + (size_t)kt * ystep;
 #pragma unroll
-    for (int i = 0; i < XL; ++i) {
-      if constexpr (YT)
-        direct_load_16(xs + xoff[i], (u32)(uintptr_t)(lptr_t)(buf + (wave * XL + i) * 1024));
-      else
-        __builtin_amdgcn_global_load_lds((gptr_t)(xs + xoff[i]), (lptr_t)(buf + (wave * XL + i) * 1024), 16, 0, 0);
-    }
+    for (int i = 0; i < XL; ++i) direct_load_16(xs + xoff[i], (u32)(uintptr_t)(lptr_t)(buf + (wave * XL + i) * 1024));
 #pragma unroll
-    for (int i = 0; i < YL; ++i) {
-      if constexpr (YT)
-        direct_load_16(ys + yoff[i], (u32)(uintptr_t)(lptr_t)(buf + T::XBYTES + (wave * YL + i) * 1024));
-      else
-        __builtin_amdgcn_global_load_lds((gptr_t)(ys + yoff[i]), (lptr_t)(buf + T::XBYTES + (wave * YL + i) * 1024),
-                                         16, 0, 0);
-    }
+    for (int i = 0; i < YL; ++i)
+      direct_load_16(ys + yoff[i], (u32)(uintptr_t)(lptr_t)(buf + T::XBYTES + (wave * YL + i) * 1024));
   };
 
   typename Op::acc_t acc[T::TX][T::TY];
@@ -180,16 +171,10 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
   auto issue_one = [&](int kt, int i) {
     char *buf = lds + (kt % NSTAGE) * T::STAGE;
     const char *xs = p.x + (size_t)kt * T::BKB, *ys = p.y + (size_t)kt * ystep;
-    if constexpr (YT) {
-      if (i < XL)
-        direct_load_16(xs + xoff[i], (u32)(uintptr_t)(lptr_t)(buf + (wave * XL + i) * 1024));
-      else
-        direct_load_16(ys + yoff[i - XL], (u32)(uintptr_t)(lptr_t)(buf + T::XBYTES + (wave * YL + (i - XL)) * 1024));
-    } else if (i < XL)
-      __builtin_amdgcn_global_load_lds((gptr_t)(xs + xoff[i]), (lptr_t)(buf + (wave * XL + i) * 1024), 16, 0, 0);
+    if (i < XL)
+      direct_load_16(xs + xoff[i], (u32)(uintptr_t)(lptr_t)(buf + (wave * XL + i) * 1024));
     else
-      __builtin_amdgcn_global_load_lds((gptr_t)(ys + yoff[i - XL]),
-                                       (lptr_t)(buf + T::XBYTES + (wave * YL + (i - XL)) * 1024), 16, 0, 0);
+      direct_load_16(ys + yoff[i - XL], (u32)(uintptr_t)(lptr_t)(buf + T::XBYTES + (wave * YL + (i - XL)) * 1024));
   };
 
   // One k-step with a fixed instruction order: every MFMA is followed by one slice of the
