@@ -175,7 +175,7 @@ extern "C" int unit_mfma_peak(int32_t f16, int32_t blocks, int32_t iters, void *
   return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "unit_mfma_peak: %s", hipGetErrorString(e));
 }
 
-extern "C" int unit_version(void) { return 104; }  // 1.4: LDS-shared convolution variants (16 KiB of zeros behind prepared int8 weights), dense on a prepared weight
+extern "C" int unit_version(void) { return 105; }  // 1.5: fp16 GEMM k-splits through a workspace or the library's static scratch; 1.4: LDS-shared convolution variants (16 KiB of zeros behind prepared int8 weights), dense on a prepared weight
 
 extern "C" const char *unit_last_error(void) { return unit::error_buf(); }
 
