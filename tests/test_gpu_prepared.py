@@ -189,27 +189,34 @@ def test_conv2d_prepared_c4_every_direct_variant(dev, oracle, monkeypatch):
     (1, 32, 5, 5, 16, 1, 1, 0),     # one k-step: k-groups beyond the first have nothing to do
     (3, 256, 7, 7, 160, 3, 2, 1),   # a long reduction over few pixels
     (1, 48, 8, 8, 32, 3, 1, 0),     # 27 taps without padding
+    (2, 16, 12, 12, 32, 3, 1, (2, 2, 2)),          # dilation 2 (third entry of the padding triple), padding 2
+    (1, 48, 10, 10, 80, 5, (2, 1), ((2, 0), 1)),   # 5 x 5 window (25 positions), anisotropic stride and padding
 ])
 def test_conv2d_prepared_every_direct_variant(dev, oracle, monkeypatch, N, C, H, W, K, ks, stride, pad):
     """u8 and fused signed form on every direct and every LDS-shared variant (ids of register-staged variants fall
     back to a direct one)."""
     from unit_amd import _lib
+    dil = 1
+    if isinstance(pad, tuple) and len(pad) == 3:    # (pad, pad, dilation)
+        pad, dil = pad[0], pad[2]
+    elif isinstance(pad, tuple) and isinstance(pad[0], tuple):  # ((pad_h, pad_w), dilation)
+        pad, dil = pad
     data = rng.uniform_u8((N, C // 16, H, W, 16), 11 * C + H)
     xs = (data ^ 0x80).view(np.int8)
     wt = rng.uniform_s8((K // 16, C // 16, ks, ks, 4, 16, 4), 5 * K + ks)
     bias = rng.uniform_s8((K,), 5).astype(np.int32) * 1001
-    ref = oracle.c_conv2d_nchwc(data, wt, stride, pad, 1)
-    ref_fused = oracle.conv2d_nchwc_int8_fused(xs, wt, bias, -7, stride, pad, 1, conv=oracle.c_conv2d_nchwc)
+    ref = oracle.c_conv2d_nchwc(data, wt, stride, pad, dil)
+    ref_fused = oracle.conv2d_nchwc_int8_fused(xs, wt, bias, -7, stride, pad, dil, conv=oracle.c_conv2d_nchwc)
     d, x, tb = _t(data, dev), _t(xs, dev), _t(bias, dev)
     p = U.prepare_conv2d_weight(_t(wt, dev))
     names = set()
     for v in range(1, _lib.load().unit_conv_variant_count() + 1):
         monkeypatch.setenv("UNIT_AMD_CONV_VARIANT", str(v))
-        out = U.conv2d_NCHWc_int8(d, p, stride, pad)
+        out = U.conv2d_NCHWc_int8(d, p, stride, pad, dil)
         torch.cuda.synchronize()
         names.add(U.last_variant())
         assert np.array_equal(out.cpu().numpy(), ref), (v, U.last_variant())
-        out = U.conv2d_NCHWc_int8_fused(x, p, tb, -7, stride, pad)
+        out = U.conv2d_NCHWc_int8_fused(x, p, tb, -7, stride, pad, dil)
         torch.cuda.synchronize()
         names.add(U.last_variant())
         assert np.array_equal(out.cpu().numpy(), ref_fused), (v, U.last_variant())
