@@ -37,7 +37,8 @@ def test_mfma_tile_f16_lane_layout(dev):
 GEMM_CASES = [(128, 768, 3072), (32, 32, 64), (100, 132, 72), (512, 4096, 256), (4096, 2048, 512), (2050, 4100, 136),
               (1024, 4096, 128), (300, 264, 96),     # both operands straight into LDS, 128 x 128 tiles, whole and ragged
               (2050, 4104, 192), (2050, 4104, 160),  # the same on 256 x 256 tiles, 128- and 64-byte stages, ragged
-              (1000, 4100, 192), (2050, 4100, 192)]  # N not a multiple of 8: b through the transposing register loader
+              (1000, 4100, 192), (2050, 4100, 192),  # N not a multiple of 8: b through the transposing register loader
+              (1, 8, 64), (3, 16, 96), (260, 8, 128)]  # one row, one 8-column chunk, one stage
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_CASES)

@@ -55,6 +55,25 @@ def test_dense_bit_exact(dev, oracle, M, N, K, packed):
     assert np.array_equal(out.cpu().numpy(), ref), U.last_variant()
 
 
+@pytest.mark.parametrize("M,N,K,kernel", [(1, 4, 64, "dma_x128_y128_k64_w2x2_r4_s1"), (5, 12, 128, "dma_x128_y128"),
+                                          (130, 132, 192, "dma_x128_y128"), (1000, 520, 320, "dma_x128_y128"),
+                                          (4096, 4096, 192, "i8denserm_x256"), (4096, 3840, 256, "i8denserm_x256")])
+def test_dense_row_major_direct_to_lds_edges(dev, oracle, M, N, K, kernel):
+    """Row-major weights with a reduction of whole 64-byte stages run the 128 x 128 all-direct tiles (in-kernel weight
+    sums): one stage only, a single row, N of one 4-column group, ragged tile edges; shapes that 256 x 256 tiles fill
+    better stay on the register pipeline.  The same on a prepared weight."""
+    a = rng.uniform_u8((M, K), 900 + M)
+    w = rng.uniform_s8((N, K), 901 + N)
+    ref = oracle.dense_logical(a, w) if M * N * K <= 1 << 28 else None
+    ta, tw = _t(a, dev), _t(w, dev)
+    out = U.dense(ta, tw)
+    assert kernel in U.last_variant(), U.last_variant()
+    if ref is None:
+        ref = (ta.double() @ tw.double().T).cpu().numpy().astype(np.int64)
+    assert np.array_equal(out.cpu().numpy(), ref), U.last_variant()
+    assert torch.equal(U.dense(ta, U.prepare_dense_weight(tw)), out), U.last_variant()
+
+
 @pytest.mark.parametrize("M,N,K", [(300, 384, 272), (37, 256, 16), (512, 640, 400), (1, 128, 48)])
 def test_dense_packed_weights_direct_to_registers(dev, oracle, monkeypatch, M, N, K):
     """The kernel variant that reads the pre-packed weight straight into MFMA fragments, forced on
