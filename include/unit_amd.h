@@ -50,7 +50,7 @@ const char *unit_last_variant(void);
 int unit_conv_variant_count(void);
 /* 1 if variant 0..count-1 takes its operands straight from global memory into MFMA fragments
  * (prepared weights or the reference's layout), 2 if it shares both operand tiles through LDS by
- * direct global -> LDS loads (int8 convolutions on prepared weights, 16-channel blocks only), 0 if
+ * direct global -> LDS loads (convolutions on prepared weights, 16-channel blocks only), 0 if
  * it stages them in LDS through registers (the reference's weight layout only), -1 if there is no
  * such variant.  For the tuner; no counterpart in the reference. */
 int unit_conv_variant_is_direct(int32_t variant);

@@ -184,7 +184,7 @@ def test_conv2d_fp16_every_variant(dev, oracle, monkeypatch, N, C, H, W, K, ks, 
     ran = set()
     for v in range(1, count + 1):
         if _lib.load().unit_conv_variant_is_direct(v - 1) == 2:
-            continue  # LDS-shared variants exist for prepared int8 weights only: the id runs the heuristic's choice here
+            continue  # LDS-shared variants exist for prepared weights only: the id runs the heuristic's choice here
         monkeypatch.setenv("UNIT_AMD_CONV_VARIANT", str(v))
         try:
             out = U.conv2d_NCHW16c_OHWI16o(ta, tb, stride, stride, "float32")

@@ -136,7 +136,7 @@ def test_tuned_tables_name_existing_variants():
             assert (npix, k, c, kh, kw, sh) not in keys, (path, row)  # one choice per shape
             keys.add((npix, k, c, kh, kw, sh))
             if path.endswith("_prepared.inc"):
-                kinds = (1, 2) if path.endswith("i8_prepared.inc") else (1,)
+                kinds = (1, 2) if path.endswith("_prepared.inc") else (1,)
                 assert L.unit_conv_variant_is_direct(variant) in kinds, (path, row)
 
 

@@ -69,11 +69,17 @@ __device__ __forceinline__ void dma_buffer_16(u32 lds_addr, u32 voff, v4i rsrc, 
                : "memory");
 }
 
-template <class S, bool SHIFT, bool Q8 = false, bool NCHW = false>
+// fp16 (Op = OpF16): a pixel and tap are 32 bytes, one k-step; the two 16-byte halves (input channels 0-7 and 8-15) take
+// the places of the int8 kernel's two taps of a k-step, so the tiling in bytes is the same.  The prepared fp16 weights
+// have no zero region behind them: their fragments come by buffer loads as well, out of range past a k-group's share.
+template <class S, bool SHIFT, bool Q8 = false, bool NCHW = false, class Op = OpI8>
 __global__ __launch_bounds__(S::NT) void conv_lds(const char *__restrict__ data, const char *__restrict__ wgt,
-                                                  const char *__restrict__ zero, typename ConvEpilogue<OpI8>::Params ep,
+                                                  const char *__restrict__ zero, typename ConvEpilogue<Op>::Params ep,
                                                   ConvGeom g, GridMap gm, int nsteps) {
-  using Op = OpI8;
+  constexpr bool F16 = !Op::kInt;
+  constexpr int ESZ = F16 ? 2 : 1;          // bytes per element
+  constexpr int SPT = F16 ? 2 : 1;          // 16-byte slots of the pixel tile per tap
+  static_assert(!F16 || (!SHIFT && !Q8), "the u8 shift and the requantised output are int8 forms");
   extern __shared__ __attribute__((aligned(16))) char lds[];
   constexpr int TX = S::TX, TY = S::TY, KG = S::KG, KS = S::KS, NST = S::NST, LW = S::LW, NM = S::NM, NF = S::NF;
   constexpr int LPK = S::LPK, LX = S::LX, LY = S::LY;
@@ -111,7 +117,7 @@ __global__ __launch_bounds__(S::NT) void conv_lds(const char *__restrict__ data,
       g.by_ohw.divmod(m, n, rem);
       g.by_ow.divmod(rem, oh, ow);
       const int ih0 = oh * g.sh - g.pt, iw0 = ow * g.sw - g.pl;
-      pixoff = (int)(n * g.img_bytes) + (ih0 * g.W + iw0) * 16;
+      pixoff = (int)(n * g.img_bytes) + (ih0 * g.W + iw0) * (16 * ESZ);
       u32 cols = 0, bits = 0;
       for (int kw = 0; kw < g.KW; ++kw) cols |= (u32)((u32)(iw0 + kw * g.dw) < (u32)g.W) << kw;
       for (int kh = 0; kh < g.KH; ++kh)
@@ -122,21 +128,24 @@ __global__ __launch_bounds__(S::NT) void conv_lds(const char *__restrict__ data,
     int p = 0;
     for (int kh = 0; kh < g.KH; ++kh)
       for (int kw = 0; kw < g.KW; ++kw, ++p)
-        mine[p * 64] = ((inside >> p) & 1u) ? (u32)(pixoff + (kh * g.dh * g.W + kw * g.dw) * 16) : kOutside;
+        mine[p * 64] = ((inside >> p) & 1u) ? (u32)(pixoff + (kh * g.dh * g.W + kw * g.dw) * (16 * ESZ)) : kOutside;
     mine[npos * 64] = kOutside;
   }
 
   const int lastkb = (ep.K - 1) >> 5;
   const u32 lane16 = (u32)lane * 16u;
-  // raw buffer over the data tensor (base, no stride, size in bytes)
-  v4i rsrc;
-  {
-    const unsigned long long base = (unsigned long long)data;
-    rsrc[0] = __builtin_amdgcn_readfirstlane((int)(u32)base);
-    rsrc[1] = __builtin_amdgcn_readfirstlane((int)((u32)(base >> 32) & 0xffffu));
-    rsrc[2] = __builtin_amdgcn_readfirstlane((int)((u32)g.N * g.img_bytes));
-    rsrc[3] = 0x00020000;
-  }
+  // raw buffers (base, no stride, size in bytes) over the data tensor and, fp16, over the weight fragments
+  auto raw_buffer = [](const char *ptr, u32 bytes) {
+    const unsigned long long base = (unsigned long long)ptr;
+    v4i r;
+    r[0] = __builtin_amdgcn_readfirstlane((int)(u32)base);
+    r[1] = __builtin_amdgcn_readfirstlane((int)((u32)(base >> 32) & 0xffffu));
+    r[2] = __builtin_amdgcn_readfirstlane((int)bytes);
+    r[3] = 0x00020000;
+    return r;
+  };
+  const v4i rsrc = raw_buffer(data, (u32)g.N * g.img_bytes);
+  const v4i wsrc = raw_buffer(wgt, (u32)(lastkb + 1) * (u32)nsteps * 1024u);
 
   // ---- this wave's direct loads of a stage, as scalar state that advances from stage to stage (they are issued
   // strictly in stage order): LX weight fragments (KiB q = wg + n * NWG of the stage's X part: k-step q / XB,
@@ -152,17 +161,22 @@ __global__ __launch_bounds__(S::NT) void conv_lds(const char *__restrict__ data,
     xsrc[n] = wgt + ((size_t)kb * nsteps + xs[n]) * 1024;
   }
   const int rg = wg % S::RG;
-  const u32 chw16 = (u32)g.H * (u32)g.W * 16u;  // bytes from one 16-channel block of an image to the next
-  const int step_ci = g.by_kh.div(g.by_kw.div(2 * KS)), step_pos = 2 * KS - step_ci * npos;  // taps per stage = ci blocks + positions
+  const u32 chw16 = (u32)g.H * (u32)g.W * (16u * ESZ);  // bytes from one 16-channel block of an image to the next
+  constexpr int TPS = 2 * KS / SPT;                      // taps per stage
+  const int step_ci = g.by_kh.div(g.by_kw.div(TPS)), step_pos = TPS - step_ci * npos;  // = ci blocks + positions
+  // the taps of this k-group end here: past it the pixel loads fetch zeros (int8: the weights there are zero and any
+  // finite data would do; fp16: zero weights times data that may hold infinities must not be formed)
+  const int tap_end = F16 ? (s1 < g.ntaps ? s1 : g.ntaps) : g.ntaps;
   int ytap[LY], ypos[LY];
   u32 yci[LY];
 #pragma unroll
   for (int n = 0; n < LY; ++n) {
-    const int t = 2 * s0 + (wg + n * S::NWG) / S::RG;
+    const int slot = 2 * s0 + (wg + n * S::NWG) / S::RG;  // 16-byte slot of the pixel tile, counted over the whole reduction
+    const int t = slot / SPT;
     const int ci = g.by_kh.div(g.by_kw.div(t));
     ytap[n] = t;
     ypos[n] = t - ci * npos;
-    yci[n] = (u32)ci * chw16;
+    yci[n] = (u32)ci * chw16 + (u32)(slot % SPT) * 16u;
   }
   const u32 *posrow = postab + rg * (npos + 1) * 64 + lane;
   u32 yvoff[LY];  // the lane's offsets of the pixel loads about to be issued, read from the position table
@@ -188,21 +202,25 @@ __global__ __launch_bounds__(S::NT) void conv_lds(const char *__restrict__ data,
   // offset of pixel load n (LX .. LW-1) out of the position table, to be read some MFMAs before the load is issued
   auto read_voff = [&](int n) {
     const int k = n - LX;
-    const int row = ytap[k] < g.ntaps ? ypos[k] : npos;
+    const int row = ytap[k] < tap_end ? ypos[k] : npos;
     yvoff[k] = posrow[row * 64];
   };
   // direct load n (0 .. LW-1) of the stage being issued; advances the load's state to the next stage
   auto issue_one = [&](int n) {
     if (n < LX) {
       const int q = wg + n * S::NWG;
-      const char *src = xs[n] < s1 ? xsrc[n] : zero;
-      dma_global_16(ring_addr + iss_off + q * 1024, lane16, src);
+      if constexpr (F16) {
+        dma_buffer_16(ring_addr + iss_off + q * 1024, xs[n] < s1 ? lane16 : kOutside, wsrc, (u32)(xsrc[n] - wgt));
+      } else {
+        const char *src = xs[n] < s1 ? xsrc[n] : zero;
+        dma_global_16(ring_addr + iss_off + q * 1024, lane16, src);
+      }
       xs[n] += KS;
       xsrc[n] += KS * 1024;
     } else {
       const int k = n - LX, q = wg + k * S::NWG;
       dma_buffer_16(ring_addr + iss_off + S::XPART + q * 1024, yvoff[k], rsrc, yci[k]);
-      ytap[k] += 2 * KS;
+      ytap[k] += TPS;
       ypos[k] += step_pos;
       yci[k] += (u32)step_ci * chw16;
       if (ypos[k] >= npos) {
@@ -212,7 +230,7 @@ __global__ __launch_bounds__(S::NT) void conv_lds(const char *__restrict__ data,
     }
   };
 
-  v16i acc[TX][TY];
+  typename Op::acc_t acc[TX][TY];
 #pragma unroll
   for (int i = 0; i < TX; ++i)
 #pragma unroll
@@ -346,7 +364,8 @@ __global__ __launch_bounds__(S::NT) void conv_lds(const char *__restrict__ data,
     }
   } else {
     // every k-group parks its partial tile; then the blocks are dealt to all waves, which add the KG partial
-    // blocks (integer sums: exact in any order) and write them
+    // blocks in k-group order (integer sums are exact in any order, fp32 sums the same from run to run) and write them
+    using out4_t = typename Op::out4_t;
     char *mine = lds + grp * (S::BX * S::BY * 4);
 #pragma unroll
     for (int i = 0; i < TX; ++i)
@@ -355,15 +374,15 @@ __global__ __launch_bounds__(S::NT) void conv_lds(const char *__restrict__ data,
         const int b = (wx * TX + i) * S::YB + wy * TY + j;
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-          *reinterpret_cast<v4i *>(mine + ((b * 4 + q) * 64 + lane) * 16) =
-              v4i{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+          *reinterpret_cast<out4_t *>(mine + ((b * 4 + q) * 64 + lane) * 16) =
+              out4_t{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
       }
     __syncthreads();
 #pragma unroll
     for (int n = 0; n < S::NBW; ++n) {
       const int b = wave + n * S::NW;
       if (b < S::NBLK) {
-        v16i total;
+        typename Op::acc_t total;
 #pragma unroll
         for (int r = 0; r < 16; ++r) total[r] = 0;
 #pragma unroll
@@ -371,7 +390,7 @@ __global__ __launch_bounds__(S::NT) void conv_lds(const char *__restrict__ data,
           const char *its = lds + w * (S::BX * S::BY * 4);
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
-            const v4i v = *reinterpret_cast<const v4i *>(its + ((b * 4 + q) * 64 + lane) * 16);
+            const out4_t v = *reinterpret_cast<const out4_t *>(its + ((b * 4 + q) * 64 + lane) * 16);
 #pragma unroll
             for (int e = 0; e < 4; ++e) total[4 * q + e] += v[e];
           }

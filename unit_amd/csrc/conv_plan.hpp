@@ -153,7 +153,7 @@ inline ConvPlan plan_conv(const unit_conv_desc *d, int npix, int kbytes, const T
   const int op = tuning_override("UNIT_AMD_CONV_PANEL");
   if (op > 0) p.panel = op;
   if (!allow_split) p.splits = 1;
-  // the LDS-shared variants exist for prepared int8 weights only: elsewhere their ids run the heuristic's choice
+  // the LDS-shared variants exist for prepared weights with 16-channel blocks only: elsewhere their ids run the heuristic's choice
   if (kConvTiles[p.variant].lds && !lds_ok) {
     const ConvPlan h = heuristic_plan(npix, d->K, kbytes, allow_split, direct_ok, d->sh * d->sw > 1, staged_too);
     p.variant = h.variant;

@@ -20,6 +20,8 @@ int conv_s8_prepared_lds(const ConvPlan &plan, const unit_conv_desc *d, const Co
 int conv_q8_prepared_lds(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
                          const char *zero, const int *addend, const int *bias, int scale, int shift, void *out,
                          hipStream_t s);  // conv_lds_q8.hip
+int conv_f16_prepared_lds(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *a, const void *w,
+                          void *out, hipStream_t s);  // conv_lds_f16.hip
 int conv_s8_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
                      const int *bias, int scale, void *out, int planar, hipStream_t s);  // conv_prepared_s8.hip
 int conv_c4_prepared(const ConvPlan &plan, const unit_conv_desc *d, const ConvGeom &g, const void *data, const void *w,
@@ -312,6 +314,7 @@ extern "C" int unit_conv2d_nchw16c_f16f32_prepared(const unit_conv_desc *d, cons
   ConvGeom g;
   if (int rc = check_prepared_conv(what, d, 32, &g, a, prepared, out)) return rc;
   const int ntable = (int)(sizeof(kTunedF16Prepared) / sizeof(kTunedF16Prepared[0])) - 1;
-  const ConvPlan p = plan_prepared(d, g, g.ntaps * 32, kTunedF16Prepared, ntable, false);
+  const ConvPlan p = plan_prepared(d, g, g.ntaps * 32, kTunedF16Prepared, ntable, false, true);
+  if (kConvTiles[p.variant].lds) return conv_f16_prepared_lds(p, d, g, a, prepared, out, static_cast<hipStream_t>(stream));
   return conv_f16_prepared(p, d, g, a, prepared, out, static_cast<hipStream_t>(stream));
 }

@@ -127,8 +127,8 @@ def tune(spec, iters=20, verbose=True, dtype="i8", prepared=False, instances=1):
             if dtype == "i8" and not prepared:
                 combos += [(n, 0) for n in (2, 4, 8, 16, 32)]
             for v in range(num_variants):
-                kind = L.unit_conv_variant_is_direct(v)  # 1 direct, 2 LDS-shared (prepared int8 weights only), 0 staged
-                if prepared and not (kind == 1 or (kind == 2 and dtype == "i8" and cb == 16)):
+                kind = L.unit_conv_variant_is_direct(v)  # 1 direct, 2 LDS-shared (prepared weights, 16-channel blocks), 0 staged
+                if prepared and not (kind == 1 or (kind == 2 and cb == 16)):
                     continue
                 if not prepared and kind == 2:
                     continue
