@@ -89,8 +89,11 @@ def tune(spec, iters=20, verbose=True, dtype="i8", prepared=False, instances=1):
                 out = torch.empty((batch, s.K // 16, oh, ow, 16), dtype=torch.float32, device=dev)
                 desc = _lib.ConvDesc(batch, cp, hp, wp, s.K, s.KH, s.KW, s.stride, s.stride, 0, 0, 0, 0, 1, 1, 16)
                 entry = L.unit_conv2d_nchw16c_f16f32
+                wt_timed = (torch.randn(wt.shape, device=dev) * 0.05).to(torch.float16)  # see the timed copies below
             if prepared:
                 from .ops import prepare_conv2d_weight
+                if dtype == "f16":
+                    wt_timed = prepare_conv2d_weight(wt_timed).buf
                 wt = prepare_conv2d_weight(wt).buf
                 entry = L.unit_conv2d_nchwc_u8s8s32_prepared if dtype == "i8" else L.unit_conv2d_nchw16c_f16f32_prepared
 
@@ -102,13 +105,36 @@ def tune(spec, iters=20, verbose=True, dtype="i8", prepared=False, instances=1):
                 n_inst = max(1, min(64, -(instances * (1 << 20)) // per + 1))
             else:
                 n_inst = instances
-            copies = [(data, wt, out)] + [(data.clone(), wt.clone(), torch.empty_like(out)) for _ in range(n_inst - 1)]
+            if dtype == "f16":
+                # copy 0 (integer-valued) is the one checked for exactness; the timed launches run on the other copies,
+                # which hold normally distributed values: the clock follows the bit activity of the operands, and on
+                # small integers an MFMA-bound layer runs up to a quarter faster than on real activations
+                n_inst = max(2, n_inst)
+                copies = [(data, wt, out)]
+                for _ in range(n_inst - 1):
+                    copies.append((torch.randn(data.shape, device=dev).to(torch.float16), wt_timed.clone(),
+                                   torch.empty_like(out)))
+                first_timed = 1
+            else:
+                copies = [(data, wt, out)] + [(data.clone(), wt.clone(), torch.empty_like(out)) for _ in range(n_inst - 1)]
+                first_timed = 0
             turn = [0]
+            timed = [False]
 
             def call():
-                d_, w_, o_ = copies[turn[0] % n_inst]
+                if timed[0]:
+                    d_, w_, o_ = copies[first_timed + turn[0] % (n_inst - first_timed)]
+                else:
+                    d_, w_, o_ = copies[turn[0] % n_inst]
                 turn[0] += 1
                 return entry(ctypes.byref(desc), d_.data_ptr(), w_.data_ptr(), o_.data_ptr(), stream)
+
+            def timed_us():
+                timed[0] = True
+                try:
+                    return time_us(call)
+                finally:
+                    timed[0] = False
 
             os.environ["UNIT_AMD_CONV_VARIANT"] = "0"
             os.environ["UNIT_AMD_CONV_SPLITK"] = "0"
@@ -120,7 +146,7 @@ def tune(spec, iters=20, verbose=True, dtype="i8", prepared=False, instances=1):
             for _ in range(n_inst):  # touch every copy once: the first launch on fresh memory is not what is being compared
                 call()
             torch.cuda.synchronize()
-            best = (time_us(call), -1, last_variant())
+            best = (timed_us(), -1, last_variant())
             default_us = best[0]
             timings = {}  # kernel name -> us, every candidate (kept in the --json dump)
             combos = [(1, 0), (1, 1), (1, 2), (1, 4)]  # (k-splits, channel tiles per panel)
@@ -150,7 +176,7 @@ def tune(spec, iters=20, verbose=True, dtype="i8", prepared=False, instances=1):
                         continue  # fewer channel tiles than the panel: same as panel 0
                     if not torch.equal(out, ref):
                         raise RuntimeError(f"variant {v} ({name}) disagrees with the default on {s.name}")
-                    us = time_us(call)
+                    us = timed_us()
                     timings[name] = round(us, 2)
                     if us < best[0]:
                         best = (us, v, name, splits, panel)
