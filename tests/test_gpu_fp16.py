@@ -70,6 +70,25 @@ def test_gemm_fp16_k_splits(dev, oracle, M, N, K):
         assert U.last_variant().endswith("_s1") and max_rel(half.cpu().numpy(), ref) <= REL_TOL
 
 
+def test_gemm_fp16_k_splits_switched_off(dev, oracle, monkeypatch):
+    """UNIT_AMD_GEMM_F16_SPLITK=1 keeps one workgroup per output tile: no fp32 atomics, so two runs give the same bits."""
+    M, N, K = 128, 768, 3072
+    a = rng.normal_f16((M, K), 141, 1.0 / np.sqrt(K))
+    b = rng.normal_f16((K, N), 142)
+    ta, tb = _t(a, dev), _t(b, dev)
+    ref = oracle.gemm_f16(a, b)
+    for operand in (tb, U.prepare_gemm_b(tb)):
+        split = U.gemm_fp16(ta, operand)
+        assert int(U.last_variant().rsplit("_s", 1)[1]) > 1, U.last_variant()
+        monkeypatch.setenv("UNIT_AMD_GEMM_F16_SPLITK", "1")
+        one = U.gemm_fp16(ta, operand)
+        assert U.last_variant().endswith("_s1"), U.last_variant()
+        again = U.gemm_fp16(ta, operand)
+        monkeypatch.delenv("UNIT_AMD_GEMM_F16_SPLITK")
+        assert torch.equal(one, again)
+        assert max_rel(one.cpu().numpy(), ref) <= REL_TOL and max_rel(split.cpu().numpy(), ref) <= REL_TOL
+
+
 PREPARED_GEMM_CASES = GEMM_CASES + [(4096, 4096, 1024), (2304, 2560, 192), (257, 260, 64), (3000, 2052, 200),
                                     (2048, 2048, 320)]  # 256 x 128 tiles: a direct to LDS, prepared b through registers
 
