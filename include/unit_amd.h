@@ -303,7 +303,9 @@ int unit_mfma_tile_f16(const void *a, const void *b, void *c, unit_stream_t stre
  * blocks * 4 * 4 * iters * 65536 (int8) or * 32768 (fp16); the caller times the launch.
  * `f16` bit 1 (values 2, 3) selects operands with random bit patterns that change from one
  * instruction to the next instead of constant ones: the chip's clocks follow its power draw, and
- * the rate it sustains depends on how many operand bits toggle.
+ * the rate it sustains depends on how many operand bits toggle.  For int8 those operands are
+ * uniform random bytes, i.e. the distribution of the 4096^3 int8 benchmark; f16 == 5 draws the
+ * fp16 operands like the fp16 benchmark does (x ~ N(0,1)/64, y ~ N(0,1)) instead of hashed bits.
  * `sink` is a 4-byte device scratch word. */
 int unit_mfma_peak(int32_t f16, int32_t blocks, int32_t iters, void *sink, unit_stream_t stream);
 

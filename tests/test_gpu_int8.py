@@ -57,11 +57,14 @@ def test_dense_bit_exact(dev, oracle, M, N, K, packed):
 
 @pytest.mark.parametrize("M,N,K,kernel", [(1, 4, 64, "dma_x128_y128_k64_w2x2_r4_s1"), (5, 12, 128, "dma_x128_y128"),
                                           (130, 132, 192, "dma_x128_y128"), (1000, 520, 320, "dma_x128_y128"),
-                                          (4096, 4096, 192, "i8denserm_x256"), (4096, 3840, 256, "i8denserm_x256")])
+                                          (4096, 4096, 192, "i8denserm_x256"), (4096, 3840, 256, "i8densedma_x256_y256"),
+                                          (2800, 4000, 384, "i8densedma_x256_y256")])
 def test_dense_row_major_direct_to_lds_edges(dev, oracle, M, N, K, kernel):
     """Row-major weights with a reduction of whole 64-byte stages run the 128 x 128 all-direct tiles (in-kernel weight
     sums): one stage only, a single row, N of one 4-column group, ragged tile edges; shapes that 256 x 256 tiles fill
-    better stay on the register pipeline.  The same on a prepared weight."""
+    better run those on the same pipeline when the reduction is a whole number of 128-byte stages (the four waves that
+    share a weight fragment divide the weight sums between them; ragged M and N edges, an odd number of stages), else
+    stay on the register pipeline.  The same on a prepared weight."""
     a = rng.uniform_u8((M, K), 900 + M)
     w = rng.uniform_s8((N, K), 901 + N)
     ref = oracle.dense_logical(a, w) if M * N * K <= 1 << 28 else None

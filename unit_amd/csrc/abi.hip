@@ -123,7 +123,8 @@ __global__ __launch_bounds__(64) void mfma_tile_f16(const char *a, const char *b
 // Register-only MFMA throughput probe in the manner of poc/vnni/micro.cc:16-51: 4 independent
 // accumulator chains per wave, no memory traffic; one workgroup of 4 waves per launch slot.
 // RANDOM: four operand pairs of hashed bits, rotated so that consecutive MFMAs see different data
-template <class Op, bool RANDOM>
+// GAUSS (fp16): the operands of the 4096^3 benchmark instead, x ~ N(0,1)/64 and y ~ N(0,1) (Box-Muller on the hashes)
+template <class Op, bool RANDOM, bool GAUSS = false>
 __global__ __launch_bounds__(256) void mfma_peak(int iters, typename Op::out_t *sink) {
   const int l = threadIdx.x;
   v4i xs[4], ys[4];
@@ -141,6 +142,16 @@ __global__ __launch_bounds__(256) void mfma_peak(int iters, typename Op::out_t *
         g ^= g >> 15; g *= 2246822519u; g ^= g >> 13;
         xs[i][d] = (int)(Op::kInt ? h : (h & 0x3fff3fffu));  // fp16: finite values below 2
         ys[i][d] = (int)(Op::kInt ? g : (g & 0x3fff3fffu));
+        if constexpr (GAUSS) {
+          auto pair = [](u32 u, float scale) {  // two normal values from one hash
+            const float r = sqrtf(-2.f * __logf(((u & 0xffffu) + 1u) * (1.f / 65537.f))) * scale;
+            const float t = (float)(u >> 16) * (6.2831853f / 65536.f);
+            const _Float16 lo = (_Float16)(r * __cosf(t)), hi = (_Float16)(r * __sinf(t));
+            return (int)((u32)__builtin_bit_cast(unsigned short, lo) | ((u32)__builtin_bit_cast(unsigned short, hi) << 16));
+          };
+          xs[i][d] = pair(h, 1.f / 64.f);
+          ys[i][d] = pair(g, 1.f);
+        }
       }
     }
   }
@@ -165,6 +176,11 @@ extern "C" int unit_mfma_peak(int32_t f16, int32_t blocks, int32_t iters, void *
   if (!sink || blocks <= 0 || iters <= 0) return fail(UNIT_E_ARG, "unit_mfma_peak: bad arguments");
   if (int rc = check_device()) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if ((f16 & 7) == 5) {  // fp16 operands distributed like the 4096^3 benchmark's
+    hipLaunchKernelGGL((mfma_peak<OpF16, true, true>), dim3(blocks), dim3(256), 0, s, iters, static_cast<float *>(sink));
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "unit_mfma_peak: %s", hipGetErrorString(e));
+  }
   switch (f16 & 3) {
     case 0: hipLaunchKernelGGL((mfma_peak<OpI8, false>), dim3(blocks), dim3(256), 0, s, iters, static_cast<int *>(sink)); break;
     case 1: hipLaunchKernelGGL((mfma_peak<OpF16, false>), dim3(blocks), dim3(256), 0, s, iters, static_cast<float *>(sink)); break;

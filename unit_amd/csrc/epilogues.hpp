@@ -23,11 +23,12 @@ struct GemmEpilogue {
   template <class T>
   static __device__ __forceinline__ void store(const Params &p, typename Op::acc_t (&acc)[T::TX][T::TY],
                                                int (&)[T::TX], int (&wsy)[T::TY], int xw0, int yw0, int lane,
-                                               int, char *, bool accumulate) {
+                                               int, char *, bool accumulate, int yrot = 0) {
+    // yrot: accumulator column j (and wsy[j]) belongs to Y block (j + yrot) % TY of the wave tile
     const int l32 = lane & 31, half = lane >> 5;
 #pragma unroll
     for (int j = 0; j < T::TY; ++j) {
-      const int n = yw0 + j * 32 + l32;
+      const int n = yw0 + ((j + yrot) % T::TY) * 32 + l32;
       if (n >= p.N) continue;
 #pragma unroll
       for (int i = 0; i < T::TX; ++i)

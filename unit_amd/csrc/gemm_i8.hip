@@ -36,7 +36,9 @@ int run_dense(const void *a, const void *w, void *c, int M, int N, int K, hipStr
 }
 
 // direct-to-LDS variant: row-major weights, K a whole number of stages.  wsum: the weight's row sums when they
-// were prepared beforehand (unit_dense_prepare_weight), else null and the kernel sums the fragments itself.
+// were prepared beforehand (unit_dense_prepare_weight), else null and the kernel sums the fragments itself -- one
+// Y block per wave where the tile has as many Y blocks per wave as waves share them (WS_Y_SPLIT: 4096^3 in 66-69 us
+// against 65 us on prepared sums; summing every fragment in every wave cost 75 us).
 template <class T, int NSTAGE, bool GIVEN = false>
 int run_dense_dma(const void *a, const void *w, void *c, int M, int N, int K, hipStream_t s, const int *wsum = nullptr,
                   int splits = 1) {
@@ -46,7 +48,8 @@ int run_dense_dma(const void *a, const void *w, void *c, int M, int N, int K, hi
   const int nk = K / T::BKB, gx = ceil_div(M, T::BX), gy = ceil_div(N, T::BY);
   constexpr int lds = NSTAGE * T::STAGE;
   static_assert(lds <= kMaxLds, "ring does not fit the LDS");
-  auto kern = mma_dma_kernel<OpI8, T, NSTAGE, Epi, GIVEN ? WS_Y_GIVEN : WS_Y, true>;
+  constexpr bool kSplitSums = !GIVEN && T::TY == T::WX && (T::TY & (T::TY - 1)) == 0 && T::TX * T::TY >= 6;
+  auto kern = mma_dma_kernel<OpI8, T, NSTAGE, Epi, GIVEN ? WS_Y_GIVEN : kSplitSums ? WS_Y_SPLIT : WS_Y, true>;
   static thread_local bool allowed = false;
   if (!allowed) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -138,6 +141,9 @@ int dense(const void *a, const void *w, void *c, int M, int N, int K, unit_strea
   if (!PACKED && K % 64 == 0 && !direct_gemm_large_tiles(M, N))
     return run_dense_dma<Tile<128, 128, 64, 2, 2>, 4>(a, w, c, M, N, K, s, nullptr,
                                                       direct_gemm_k_splits("UNIT_AMD_DENSE_SPLITK", M, N, K));
+  // the large tiles on the same pipeline: the four waves that share a weight fragment divide the weight sums
+  if (!PACKED && K % 128 == 0 && direct_gemm_large_tiles(M, N))
+    return run_dense_dma<Tile<256, 256, 128, 4, 2>, 2>(a, w, c, M, N, K, s);
   if (M >= 256 && N >= 256 && tiles_big >= 128)
     return K % 128 ? run_dense<Tile<256, 256, 128, 2, 4>, PACKED>(a, w, c, M, N, K, s)
                    : run_dense<Tile<256, 256, 128, 2, 4>, PACKED, false>(a, w, c, M, N, K, s);

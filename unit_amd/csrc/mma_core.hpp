@@ -139,7 +139,7 @@ struct GridMap {
   }
 };
 
-enum { WS_NONE = 0, WS_X = 1, WS_Y = 2, WS_Y_GIVEN = 3 };  // weight sums: none, summed in the kernel (X / Y rows), read from memory
+enum { WS_NONE = 0, WS_X = 1, WS_Y = 2, WS_Y_GIVEN = 3, WS_Y_SPLIT = 4 };  // weight sums: none, summed in the kernel (X / Y rows), read from memory, summed in the kernel one Y block per wave
 
 // The kernel.  XL / YL stage the operand tiles, Epi writes the accumulators.
 // WS selects which operand is the s8 weight whose per-row byte sums are accumulated on the side

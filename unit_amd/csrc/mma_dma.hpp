@@ -35,10 +35,22 @@ typedef short v4s __attribute__((ext_vector_type(4)));
 // for a fragment read becomes a wait for all of them (lgkmcnt(0) at the head of every k-step), and it makes the
 // transposing LDS read wait for all direct loads in flight (it cannot tell which LDS bytes a load fills), which
 // undoes the ring.  Loads issued this way are invisible to it, so the kernel's own vmcnt waits order them alone.
+// m0 is a register the compiler reserves: it never keeps a value in it across statements (it writes m0 right before
+// each instruction of its own that reads it), so the statement may overwrite it; naming it as a clobber is rejected
+// ("clobber list contains reserved registers").
 __device__ __forceinline__ void direct_load_16(const void *src, u32 lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
                :
                : "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(src)
+               : "memory");
+}
+// The same with the address as a wave-uniform base (SGPR pair) plus a 32-bit lane offset, and the LDS position in an
+// SGPR: no vector instruction is spent on addresses, and no vector -> scalar hand-over sits in front of the load.
+// (Cache-policy bits on these loads were measured at 4096^3: sc0 / sc1 within noise, nt 6-15 % slower.)
+__device__ __forceinline__ void direct_load_16s(const void *sbase, u32 voff, u32 lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(sbase)
                : "memory");
 }
 
@@ -52,7 +64,9 @@ template <class Op, class T, int NSTAGE, class Epi, int WS, bool XOR_X, bool YT 
 __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Epi::Params ep, int nk, GridMap gm) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   const int t = threadIdx.x;
-  const int lane = t & 63, wave = t >> 6;
+  const int lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);  // wave-uniform: LDS positions of the direct loads stay scalar
+  const u32 ring_addr = (u32)(uintptr_t)(lptr_t)lds;
   const int wx = wave % T::WX, wy = wave / T::WX;
   const int l32 = lane & 31, half = lane >> 5;
   constexpr int KK = T::BKB / 32, CPR = T::CPR, NW = T::NT / 64;
@@ -65,6 +79,12 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
   constexpr int CPRY = T::BY / 8, RPLY = 64 / CPRY;  // YT: chunks per k row, k rows per wave-level load
   static_assert(!YT || (CPRY >= 16 && CPRY <= 64 && (T::BKB / 2) % (RPLY * NW) == 0 && YL == T::BKB / 2 / RPLY / NW &&
                         WS == WS_NONE && !XOR_X), "transposed-Y tile shape");
+  // WS_Y_SPLIT: the WX waves that read the same Y fragments (same wy) share the weight sums: wave wx reads the Y
+  // blocks of its tile rotated by wx, so the block it sums is always its fragment 0 (four v_dot4 per k-step and wave
+  // instead of 4 * TY), and the waves exchange their sums through LDS after the loop.
+  constexpr bool SPLIT = WS == WS_Y_SPLIT;
+  static_assert(!SPLIT || (T::TY == T::WX && (T::TY & (T::TY - 1)) == 0 && T::TX * T::TY >= 6 && !YT),
+                "split weight sums: one Y block per wave of a row of waves");
 
   int bx, by, split;
   gm.locate(blockIdx.x, bx, by, split);
@@ -103,14 +123,17 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
     }
   }
 
+  // load i of stage kt's LPS loads of this wave, into ring buffer `slot`
+  auto issue_one = [&](int kt, int slot, int i) {
+    const u32 buf = ring_addr + (u32)(slot * T::STAGE);
+    if (i < XL)
+      direct_load_16s(p.x + (size_t)kt * T::BKB, xoff[i], buf + (wave * XL + i) * 1024);
+    else
+      direct_load_16s(p.y + (size_t)kt * ystep, yoff[i - XL], buf + T::XBYTES + (wave * YL + (i - XL)) * 1024);
+  };
   auto issue = [&](int kt) {
-    char *buf = lds + (kt % NSTAGE) * T::STAGE;
-    const char *xs = p.x + (size_t)kt * T::BKB, *ys = p.y + (size_t)kt * ystep;
 #pragma unroll
-    for (int i = 0; i < XL; ++i) direct_load_16(xs + xoff[i], (u32)(uintptr_t)(lptr_t)(buf + (wave * XL + i) * 1024));
-#pragma unroll
-    for (int i = 0; i < YL; ++i)
-      direct_load_16(ys + yoff[i], (u32)(uintptr_t)(lptr_t)(buf + T::XBYTES + (wave * YL + i) * 1024));
+    for (int i = 0; i < LPS; ++i) issue_one(kt, kt % NSTAGE, i);
   };
 
   typename Op::acc_t acc[T::TX][T::TY];
@@ -127,8 +150,12 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
   for (int j = 0; j < T::TY; ++j) wsy[j] = 0;
 
   const int xrow = wx * (T::TX * 32) + l32, yrow = wy * (T::TY * 32) + l32;
-  const int xsw = swz<T::BKB>(xrow), ysw = swz<T::BKB>(yrow);
+  const int xsw = swz<T::BKB>(xrow), ysw = swz<T::BKB>(yrow);  // the swizzle repeats every 16 rows
   const int xbase = xrow * T::BKB, ybase = T::XBYTES + yrow * T::BKB;
+  const int yrot = SPLIT ? wx : 0;
+  int yblk[T::TY];  // fragment j of this wave is Y block (j + yrot) % TY of the wave tile
+#pragma unroll
+  for (int j = 0; j < T::TY; ++j) yblk[j] = ybase + ((j + yrot) % T::TY) * 32 * T::BKB;
 
   // YT: byte offset, inside the Y tile, of what this lane hands to the transposing reads of fragment j at k-step 0,
   // read 0: k row 8 * half + (lane % 16) / 4, columns 32 j + 16 * ((lane / 16) % 2) + 4 * (lane % 4) .. + 3
@@ -158,7 +185,7 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
         const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((trptr_t)(src + 4 * (T::BY * 2)));
         yf[s][idx - 1] = __builtin_bit_cast(v4i, (v8s)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
       } else {
-        yf[s][idx - 1] = *reinterpret_cast<const v4i *>(stage + ybase + (idx - 1) * 32 * T::BKB + cy);
+        yf[s][idx - 1] = *reinterpret_cast<const v4i *>(stage + (SPLIT ? yblk[idx - 1] : ybase + (idx - 1) * 32 * T::BKB) + cy);
       }
     }
     else
@@ -168,22 +195,13 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
 #pragma unroll
     for (int i = 0; i < T::TX + T::TY; ++i) load_one(stage, kk, s, i);
   };
-  auto issue_one = [&](int kt, int i) {
-    char *buf = lds + (kt % NSTAGE) * T::STAGE;
-    const char *xs = p.x + (size_t)kt * T::BKB, *ys = p.y + (size_t)kt * ystep;
-    if (i < XL)
-      direct_load_16(xs + xoff[i], (u32)(uintptr_t)(lptr_t)(buf + (wave * XL + i) * 1024));
-    else
-      direct_load_16(ys + yoff[i - XL], (u32)(uintptr_t)(lptr_t)(buf + T::XBYTES + (wave * YL + (i - XL)) * 1024));
-  };
-
   // One k-step with a fixed instruction order: every MFMA is followed by one slice of the
   // step's other work (a fragment read for the next step, a direct load for a later stage, the
   // u8 -> s8 shift of the next X fragment, one weight-sum dot) and a scheduling fence, because
   // with one wave per SIMD only instructions placed between two MFMAs overlap with them.
   //   s: fragment slot consumed;  rd_stage/rd_kk: where the next step's fragments come from
   //   (nullptr: none);  issue_kt >= 0: stage to fetch with direct loads.
-  auto step = [&](int s, const char *rd_stage, int rd_kk, int issue_kt, auto has_read, auto has_issue) {
+  auto step = [&](int s, const char *rd_stage, int rd_kk, int issue_kt, int issue_slot, auto has_read, auto has_issue) {
     constexpr int NM = T::TX * T::TY, NF = T::TX + T::TY;
     if constexpr (XOR_X) xf[s][0] ^= (int)0x80808080;
 #pragma unroll
@@ -194,10 +212,13 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
         if (m < NF) load_one(rd_stage, rd_kk, s ^ 1, m);
       }
       if constexpr (decltype(has_issue)::value) {
-        if (m >= NM - LPS) issue_one(issue_kt, m - (NM - LPS));
+        if (m >= NM - LPS) issue_one(issue_kt, issue_slot, m - (NM - LPS));
       }
       if constexpr (XOR_X) {
         if (j == T::TY - 1 && i + 1 < T::TX) xf[s][i + 1] ^= (int)0x80808080;
+      }
+      if constexpr (SPLIT) {
+        if (m >= 2 && m < 6) wsy[0] = __builtin_amdgcn_sdot4(yf[s][0][m - 2], 0x01010101, wsy[0], false);
       }
       if constexpr (WS == WS_Y) {
         // TY fragments x 4 dwords spread over the step's MFMAs, DPM dots after each
@@ -217,12 +238,15 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
   // One stage.  ISSUE: stage kt + NSTAGE exists and is fetched into the buffer this stage
   // frees; STEADY: NSTAGE-1 younger stages are in flight when the barrier is reached (else
   // wait for everything); NEXT: stage kt + 1 exists.
-  auto stage = [&](int kt, auto issue_next, auto steady, auto next) {
-    const char *cur = lds + (kt % NSTAGE) * T::STAGE;
+  // slot: the ring buffer of stage kt (kt % NSTAGE; a constant in the unrolled steady-state loop, so that every LDS
+  // address of a stage is a register plus an immediate)
+  auto stage = [&](int kt, int slot, auto issue_next, auto steady, auto next) {
+    const char *cur = lds + slot * T::STAGE;
+    const int slot_next = slot + 1 == NSTAGE ? 0 : slot + 1;
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
       if (kk + 1 < KK) {
-        step(kk & 1, cur, kk + 1, -1, std::true_type{}, std::false_type{});
+        step(kk & 1, cur, kk + 1, -1, 0, std::true_type{}, std::false_type{});
       } else {
         // stage kt+1 must have landed; stages kt+2 .. kt+NSTAGE-1 may stay in flight
         if constexpr (decltype(steady)::value)
@@ -233,7 +257,7 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
         // every wave has read stage kt: its buffer takes stage kt + NSTAGE
-        step(kk & 1, lds + ((kt + 1) % NSTAGE) * T::STAGE, 0, kt + NSTAGE, next, issue_next);
+        step(kk & 1, lds + slot_next * T::STAGE, 0, kt + NSTAGE, slot, next, issue_next);
       }
     }
   };
@@ -253,13 +277,27 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
   load_frags(lds, 0, 0);
 
   int kt = 0;
-  for (; kt + NSTAGE < nk; ++kt) stage(kt, yes{}, yes{}, yes{});
-  for (; kt + 1 < nk; ++kt) stage(kt, no{}, no{}, yes{});
-  if (kt < nk) stage(kt, no{}, no{}, no{});
+  for (; kt + 2 * NSTAGE <= nk; kt += NSTAGE) {  // steady state, unrolled by the ring: kt % NSTAGE == 0 here
+#pragma unroll
+    for (int s = 0; s < NSTAGE; ++s) stage(kt + s, s, yes{}, yes{}, yes{});
+  }
+  for (; kt + NSTAGE < nk; ++kt) stage(kt, kt % NSTAGE, yes{}, yes{}, yes{});
+  for (; kt + 1 < nk; ++kt) stage(kt, kt % NSTAGE, no{}, no{}, yes{});
+  if (kt < nk) stage(kt, kt % NSTAGE, no{}, no{}, no{});
 
   if constexpr (WS == WS_Y) {
 #pragma unroll
     for (int j = 0; j < T::TY; ++j) wsy[j] += __shfl_xor(wsy[j], 32);
+  }
+  if constexpr (SPLIT) {
+    // The ring buffer that the last stage does not use is free once its barrier is passed: the waves leave the sums
+    // of their blocks there, [wy][block][32 rows], and pick up all TY blocks of their row of waves.
+    int *sums = reinterpret_cast<int *>(lds + ((nk + NSTAGE - 2) % NSTAGE) * T::STAGE);
+    const int part = wsy[0] + __shfl_xor(wsy[0], 32);
+    if (half == 0) sums[(wy * T::TY + yrot) * 32 + l32] = part;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < T::TY; ++j) wsy[j] = sums[(wy * T::TY + ((j + yrot) % T::TY)) * 32 + l32];
   }
   if constexpr (WS == WS_Y_GIVEN) {
 #pragma unroll
@@ -272,7 +310,7 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
     Epi::template store<T>(ep, acc, wsx, wsy, x0 + wx * (T::TX * 32), y0 + wy * (T::TY * 32), lane, wave, lds, split);
   else
     Epi::template store<T>(ep, acc, wsx, wsy, x0 + wx * (T::TX * 32), y0 + wy * (T::TY * 32), lane, wave, lds,
-                           gm.splits > 1);
+                           gm.splits > 1, yrot);
 }
 
 }  // namespace unit
