@@ -3,6 +3,7 @@
 #include <stdlib.h>
 
 #include "host.hpp"
+#include "trace.hpp"
 #include "loaders.hpp"
 
 namespace unit {
@@ -190,6 +191,17 @@ extern "C" int unit_mfma_peak(int32_t f16, int32_t blocks, int32_t iters, void *
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "unit_mfma_peak: %s", hipGetErrorString(e));
 }
+
+#ifdef UNIT_TRACE_BUILD
+// the timeline build only (make trace): the device buffer the instrumented kernels write their stamps to
+namespace unit {
+static unsigned long long *g_trace_buffer = nullptr;
+unsigned long long *trace_buffer() { return g_trace_buffer; }
+}  // namespace unit
+extern "C" void unit_trace_set(void *device_buffer) { unit::g_trace_buffer = static_cast<unsigned long long *>(device_buffer); }
+extern "C" int unit_trace_words(void) { return unit::kTraceWords; }
+extern "C" int unit_trace_waves(void) { return unit::kTraceWaves; }
+#endif
 
 extern "C" int unit_version(void) { return 105; }  // 1.5: fp16 GEMM k-splits through a workspace or the library's static scratch; 1.4: LDS-shared convolution variants (16 KiB of zeros behind prepared int8 weights), dense on a prepared weight
 

@@ -42,6 +42,7 @@
 #pragma once
 #include "epilogues.hpp"
 #include "loaders.hpp"
+#include "trace.hpp"
 
 namespace unit {
 
@@ -112,7 +113,7 @@ __device__ __forceinline__ void store_block(const typename ConvEpilogue<Op>::Par
 #pragma unroll
       for (int e = 0; e < 4; ++e)
         if (c0 + 8 * q + 4 * half + e < p.planar && m < p.npix)
-          __builtin_nontemporal_store(v[e], dst + (size_t)(8 * q + e) * p.ohw);
+          store_result(dst + (size_t)(8 * q + e) * p.ohw, v[e]);
     }
     return;
   }
@@ -126,19 +127,19 @@ __device__ __forceinline__ void store_block(const typename ConvEpilogue<Op>::Par
     *reinterpret_cast<out4_t *>(scratch + l32 * kPitch + (8 * q + 4 * half) * 4) = v;
   }
   const int ko_planes = p.K >> 4;
+  const __amdgpu_buffer_rsrc_t obuf = result_buffer(p.out);
 #pragma unroll
   for (int it = 0; it < 2; ++it) {
     const int m = m0 + it * 16 + rp;
     int n, pix;
     p.by_ohw.divmod(m, n, pix);
-    const size_t obase = ((size_t)n * ko_planes * p.ohw + pix) * 16 + piece * 4;
+    const u32 obase = ((u32)(n * ko_planes) * (u32)p.ohw + (u32)pix) * 16u + (u32)piece * 4u;  // in elements
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int c = c0 + h * 16;
       const out4_t v = *reinterpret_cast<const out4_t *>(scratch + (it * 16 + rp) * kPitch + h * 64 + piece * 16);
       if (c < p.K && m < p.npix)
-        __builtin_nontemporal_store(
-            v, reinterpret_cast<out4_t *>(reinterpret_cast<out_t *>(p.out) + obase + (size_t)(c >> 4) * p.ohw * 16));
+        store_result16(obuf, (obase + (u32)(c >> 4) * (u32)p.ohw * 16u) * (u32)sizeof(out_t), v);
     }
   }
 }
@@ -201,16 +202,19 @@ __device__ __forceinline__ void store_block_q8(const typename ConvEpilogue<Op>::
   if (c < p.K && m < p.npix) {
     int n, pix;
     p.by_ohw.divmod(m, n, pix);
-    char *dst = static_cast<char *>(p.out) + (((size_t)n * (p.K >> 4) + (c >> 4)) * p.ohw + pix) * 16;
-    __builtin_nontemporal_store(row, reinterpret_cast<v4i *>(dst));
+    store_result16(result_buffer(p.out), (((u32)(n * (p.K >> 4)) + (u32)(c >> 4)) * (u32)p.ohw + (u32)pix) * 16u, row);
   }
 }
 
 template <class Op, class S, bool SHIFT, bool PREP = false, bool C4 = false, bool Q8 = false, bool NCHW = false>
 __global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !C4 ? S::kMinWavesPerSimd : 1))) void conv_direct(const char *__restrict__ data, const char *__restrict__ wgt,
-                                                     typename ConvEpilogue<Op>::Params ep, ConvGeom g, GridMap gm) {
+                                                     typename ConvEpilogue<Op>::Params ep, ConvGeom g, GridMap gm
+                                                     UNIT_TRACE(, unsigned long long *trace_buf)) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   constexpr int TX = S::TX, TY = S::TY, KG = S::KG, D = S::D;
+  // timeline: 0 entry, 1 arguments fetched, 2 tables and per-lane window state built, 3 past the barrier, 4 ring
+  // issued, 5 reduction done (accumulators complete), 6 k-groups summed, 7 stores issued and acknowledged
+  UNIT_TRACE(WaveTrace tr; tr.mark(0);)
   {
     // Touch every 64-byte line of the 260 bytes of kernel arguments at once: the compiler fetches the arguments
     // where it first needs them, in three dependent rounds of scalar loads before the first operand fetch.
@@ -218,6 +222,7 @@ __global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !
     const int w0 = ka[0], w1 = ka[16], w2 = ka[32], w3 = ka[48], w4 = ka[64];
     asm volatile("" ::"s"(w0), "s"(w1), "s"(w2), "s"(w3), "s"(w4));
   }
+  UNIT_TRACE(tr.mark(1);)
   constexpr bool kInt = Op::kInt;
   constexpr int TAPB = C4 ? 4 : (kInt ? 16 : 32);  // bytes of one pixel and tap
   constexpr int WTAP = kInt ? 256 : 512;           // bytes of one tap of a 16-channel weight block
@@ -463,7 +468,9 @@ __global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !
     if constexpr (D > 7) f(std::integral_constant<int, 7>{});
   };
 
+  UNIT_TRACE(asm volatile("s_nop 0" ::"v"(xoff[0]), "v"(pixoff[0]), "v"(inside[0])); tr.mark(2);)
   __syncthreads();  // tap table (and the zeroed sums) visible
+  UNIT_TRACE(tr.mark(3);)
 
   const int s0 = nsteps * wave / KG, s1 = nsteps * (wave + 1) / KG;
   if (s0 < s1) {
@@ -474,6 +481,7 @@ __global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !
       fetch(u);
       __builtin_amdgcn_sched_barrier(0);
     });
+    UNIT_TRACE(tr.mark(4);)
     int s = s0;
     // while more than D k-steps remain: consume a round and fetch the next one (in the last round fewer than D
     // k-steps are new; the surplus fetches repeat the wave's last k-step)
@@ -490,6 +498,7 @@ __global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !
     });
   }
 
+  UNIT_TRACE(asm volatile("s_nop 0" ::"v"(acc[TX - 1][TY - 1][15])); tr.mark(5);)
   // the two 32-lane halves hold the weight sums of the two taps of every k-step
   if constexpr (SHIFT && !PREP) {
 #pragma unroll
@@ -532,6 +541,7 @@ __global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !
         __hip_atomic_fetch_add(wsum + i * 32 + l32, wsx[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
     __syncthreads();
+    UNIT_TRACE(tr.mark(6);)
     for (int b = wave; b < TX * TY; b += KG) {
       const int i = b / TY, j = b - i * TY;
       v16i total;
@@ -589,6 +599,7 @@ __global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !
       }
     }
   }
+  UNIT_TRACE(__builtin_amdgcn_s_waitcnt(0x0F70); tr.mark(7); tr.flush(trace_buf, blockIdx.x * KG + wave);)
 }
 
 }  // namespace unit

@@ -21,19 +21,15 @@ int run_direct(const char *what, const char *tag, const unit_conv_desc *d, const
     lds_allowed = kMaxLds;
   }
   typename ConvEpilogue<Op>::Params ep{out, d->K, g.by_ohw.d, g.npix, g.by_ohw, bias, scale, bias2, shift, planar};
-  GridMap gm;
-  gm.gx = ceil_div(d->K, S::BX);
-  gm.gy = ceil_div(g.npix, S::BY);
-  const int panel = plan.panel > 0 && plan.panel < gm.gx ? plan.panel : 0;
-  gm.ph = panel ? panel : gm.gx;
-  gm.splits = 1;
-  gm.total = gm.gx * gm.gy;
+  const int gx = ceil_div(d->K, S::BX), gy = ceil_div(g.npix, S::BY);
+  const int panel = plan.panel > 0 && plan.panel < gx ? plan.panel : 0;
+  const GridMap gm = GridMap::make(gx, gy, panel ? panel : gx, 1);
   char tail[16] = "";
   if (panel) snprintf(tail, sizeof tail, "_r%d", panel);
   set_variant("%s_x%d_y%d_g%d_d%d%s%s%s_s1", tag, S::BX, S::BY, S::KG, S::D,
               S::kFourWaves ? "w4" : "", S::PAD ? "" : "n", tail);
   hipLaunchKernelGGL(kern, dim3(gm.total), dim3(S::NT), lds, s, static_cast<const char *>(data),
-                     static_cast<const char *>(w), ep, g, gm);
+                     static_cast<const char *>(w), ep, g, gm UNIT_TRACE(, trace_buffer()));
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "%s: launch: %s", what, hipGetErrorString(e));
   return UNIT_OK;

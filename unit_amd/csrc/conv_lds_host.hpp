@@ -23,13 +23,9 @@ int run_lds(const char *what, const char *tag, const unit_conv_desc *d, const Co
     allowed = true;
   }
   typename ConvEpilogue<Op>::Params ep{out, d->K, g.OH * g.OW, g.npix, g.by_ohw, bias, scale, bias2, shift, planar};
-  GridMap gm;
-  gm.gx = ceil_div(d->K, S::BX);
-  gm.gy = ceil_div(g.npix, S::BY);
-  const int panel = plan.panel > 0 && plan.panel < gm.gx ? plan.panel : 0;
-  gm.ph = panel ? panel : gm.gx;
-  gm.splits = 1;
-  gm.total = gm.gx * gm.gy;
+  const int gx = ceil_div(d->K, S::BX), gy = ceil_div(g.npix, S::BY);
+  const int panel = plan.panel > 0 && plan.panel < gx ? plan.panel : 0;
+  const GridMap gm = GridMap::make(gx, gy, panel ? panel : gx, 1);
   char tail[16] = "";
   if (panel) snprintf(tail, sizeof tail, "_r%d", panel);
   set_variant("%s_x%d_y%d_w%dx%d_g%d_k%d_r%d%s_s1", tag, S::BX, S::BY, S::WX, S::WY, S::KG, S::KS, S::NST, tail);

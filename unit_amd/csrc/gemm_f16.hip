@@ -33,10 +33,10 @@ int run_gemm_f16_bt_dma(const void *a, const void *bt, void *c, int M, int N, in
     const size_t n16 = (size_t)M * N * 4 / 16;
     hipLaunchKernelGGL(zero_fill, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, s, static_cast<v4i *>(c), n16);
   }
-  GridMap gm{gx, gy, gx < 4 ? gx : 4, splits, gx * gy * splits};
+  const GridMap gm = GridMap::make(gx, gy, gx < 4 ? gx : 4, splits);
   set_variant("f16gemmbt_dma_x%d_y%d_k%d_w%dx%d_r%d%s_s%d", T::BX, T::BY, T::BKB, T::WX, T::WY, NSTAGE, OUT_F16 ? "_h" : "",
               splits);
-  hipLaunchKernelGGL(kern, dim3(gm.total), dim3(T::NT), lds, s, p, ep, nk, gm);
+  hipLaunchKernelGGL(kern, dim3(gm.total), dim3(T::NT), lds, s, p, ep, nk, gm UNIT_TRACE(, trace_buffer()));
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "unit_gemm_f16_prepared: launch: %s", hipGetErrorString(e));
 }
@@ -63,9 +63,9 @@ int run_gemm_f16_dma_tr(const char *what, const char *tag, const void *a, const 
     const size_t n16 = (size_t)M * N * 4 / 16;
     hipLaunchKernelGGL(zero_fill, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, s, static_cast<v4i *>(zero), n16);
   }
-  GridMap gm{gx, gy, gx < 4 ? gx : 4, splits, gx * gy * splits};
+  const GridMap gm = GridMap::make(gx, gy, gx < 4 ? gx : 4, splits);
   set_variant("f16gemm_%s_x%d_y%d_k%d_w%dx%d_r%d_s%d", tag, T::BX, T::BY, T::BKB, T::WX, T::WY, NSTAGE, splits);
-  hipLaunchKernelGGL(kern, dim3(gm.total), dim3(T::NT), lds, s, p, ep, nk, gm);
+  hipLaunchKernelGGL(kern, dim3(gm.total), dim3(T::NT), lds, s, p, ep, nk, gm UNIT_TRACE(, trace_buffer()));
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "%s: launch: %s", what, hipGetErrorString(e));
 }
@@ -95,7 +95,7 @@ int run_gemm_f16_hybrid(const void *a, const void *b, void *c, int M, int N, int
     if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "unit_gemm_f16: hipFuncSetAttribute: %s", hipGetErrorString(e));
     allowed = true;
   }
-  GridMap gm{gx, gy, gx < 4 ? gx : 4, 1, gx * gy};
+  const GridMap gm = GridMap::make(gx, gy, gx < 4 ? gx : 4, 1);
   set_variant("f16gemm_hybrid_x%d_y%d_k%d_w%dx%d%s", T::BX, T::BY, T::BKB, T::WX, T::WY, OUT_F16 ? "_h" : "");
   hipLaunchKernelGGL(kern, dim3(gm.total), dim3(T::NT), lds, s, p, yp, ep, nk, gm);
   hipError_t e = hipGetLastError();

@@ -62,10 +62,10 @@ int run_dense_dma(const void *a, const void *w, void *c, int M, int N, int K, hi
     const size_t n16 = (size_t)M * N * 4 / 16;
     hipLaunchKernelGGL(zero_fill, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, s, static_cast<v4i *>(c), n16);
   }
-  GridMap gm{gx, gy, gx < 4 ? gx : 4, splits, gx * gy * splits};
+  const GridMap gm = GridMap::make(gx, gy, gx < 4 ? gx : 4, splits);
   set_variant("i8dense%sdma_x%d_y%d_k%d_w%dx%d_r%d_s%d", GIVEN ? "prep_" : "", T::BX, T::BY, T::BKB, T::WX, T::WY, NSTAGE,
               splits);
-  hipLaunchKernelGGL(kern, dim3(gm.total), dim3(T::NT), lds, s, p, ep, nk, gm);
+  hipLaunchKernelGGL(kern, dim3(gm.total), dim3(T::NT), lds, s, p, ep, nk, gm UNIT_TRACE(, trace_buffer()));
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? UNIT_OK : fail(UNIT_E_LAUNCH, "unit_dense_u8s8s32: launch: %s", hipGetErrorString(e));
 }
@@ -90,7 +90,7 @@ int run_dense_mixed(const void *a, const void *wp, void *c, int M, int N, int K,
     if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "%s: hipFuncSetAttribute: %s", what, hipGetErrorString(e));
     allowed = true;
   }
-  GridMap gm{gx, gy, gx < 4 ? gx : 4, 1, gx * gy};
+  const GridMap gm = GridMap::make(gx, gy, gx < 4 ? gx : 4, 1);
   set_variant("i8densepk_direct_x%d_y%d_k%d_w%d_s1", T::BX, T::BY, T::BKB, T::NT / 64);
   hipLaunchKernelGGL(kern, dim3(gm.total), dim3(T::NT), lds, s, xp, static_cast<const char *>(wp), N, K / 4, ep, nk, gm);
   hipError_t e = hipGetLastError();

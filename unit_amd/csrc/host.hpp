@@ -174,12 +174,7 @@ int launch_mma(const typename XL::Params &xp, const typename YL::Params &yp, con
     hipLaunchKernelGGL(zero_fill, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, stream,
                        static_cast<v4i *>(out), n16);
   }
-  GridMap gm;
-  gm.gx = gx;
-  gm.gy = gy;
-  gm.ph = ph < 1 ? 1 : (ph > gx ? gx : ph);
-  gm.splits = splits;
-  gm.total = gx * gy * splits;
+  const GridMap gm = GridMap::make(gx, gy, ph, splits);
   hipLaunchKernelGGL(kern, dim3(gm.total), dim3(T::NT), lds, stream, xp, yp, ep, nk, gm);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(UNIT_E_LAUNCH, "%s: launch: %s", what, hipGetErrorString(e));

@@ -28,6 +28,33 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef unsigned int u32;
 
+// Result stores.  Results are written once and never read back by the kernel that writes them, so they are stored at
+// agent scope (sc1): the line goes through the XCD's L2 to memory at once instead of waiting there, dirty, for the
+// write-back at the end of the kernel.  Measured on a 102.8 MB fill: 15.05 us (6.83 TB/s) against 16.44 us for plain
+// stores and 16.56 us for non-temporal ones; sc0 changes nothing, nt on top of sc1 loses half of the gain.
+// Scalars go out as relaxed agent-scope atomic stores (global_store_dword / _short ... sc1); 16-byte vectors as raw
+// buffer stores with the sc1 policy bit, at a 32-bit byte offset from the tensor's base (tensors stay below 2^31
+// bytes).  Both are instructions the compiler knows, so its hazard and wait-count passes see them.
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t result_buffer(void *base) {
+  return __builtin_amdgcn_make_buffer_rsrc(base, 0, -1, 0x00020000);
+}
+template <class V>
+__device__ __forceinline__ void store_result16(__amdgpu_buffer_rsrc_t buf, u32 byte_offset, V v) {
+  static_assert(sizeof(V) == 16, "a 16-byte vector");
+  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), buf, (int)byte_offset, 0, 16 /* sc1 */);
+}
+__device__ __forceinline__ void store_result(int *p, int v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_result(float *p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_result(_Float16 *p, _Float16 v) {
+  __hip_atomic_store(reinterpret_cast<unsigned short *>(p), __builtin_bit_cast(unsigned short, v), __ATOMIC_RELAXED,
+                     __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // 4-byte-aligned views for gathers whose address is only dword aligned
 typedef int v4i_a4 __attribute__((ext_vector_type(4), aligned(4)));
 
@@ -123,19 +150,44 @@ struct Tile {
 // compact patch of the grid.  The k-splits of one tile are adjacent logical ids.
 struct GridMap {
   int gx, gy, ph, splits, total;  // total = gx * gy * splits
+  // dividers by splits, by ph * gy (tiles per panel), by ph and by the height of the last panel: the walk costs a
+  // few multiplies instead of three integer divisions at the head of every workgroup
+  FastDiv by_splits, by_panel, by_ph, by_last;
+  __host__ static GridMap make(int gx, int gy, int ph, int splits) {
+    GridMap m;
+    m.gx = gx;
+    m.gy = gy;
+    m.ph = ph < 1 ? 1 : (ph > gx ? gx : ph);
+    m.splits = splits < 1 ? 1 : splits;
+    m.total = gx * gy * m.splits;
+    m.by_splits = FastDiv::make(m.splits);
+    m.by_panel = FastDiv::make(m.ph * gy);
+    m.by_ph = FastDiv::make(m.ph);
+    m.by_last = FastDiv::make(gx % m.ph ? gx % m.ph : m.ph);
+    return m;
+  }
   __device__ __forceinline__ void locate(int bid, int &bx, int &by, int &split) const {
     constexpr int NXCD = 8;
     int per = total / NXCD, rem = total % NXCD;
     int xcd = bid % NXCD, idx = bid / NXCD;
     int logical = xcd * per + (xcd < rem ? xcd : rem) + idx;
-    split = logical % splits;
-    logical /= splits;
-    int panel_sz = ph * gy;
-    int panel = logical / panel_sz, within = logical - panel * panel_sz;
+    split = 0;
+    if (splits > 1) {
+      int q;
+      by_splits.divmod(logical, q, split);
+      logical = q;
+    }
+    const int panel = by_panel.div(logical), within = logical - panel * (ph * gy);
     int rows = gx - panel * ph;
-    rows = rows < ph ? rows : ph;
-    bx = panel * ph + within % rows;
-    by = within / rows;
+    const bool full = rows >= ph;
+    rows = full ? ph : rows;
+    FastDiv r;
+    r.mul = full ? by_ph.mul : by_last.mul;
+    r.shift = full ? by_ph.shift : by_last.shift;
+    r.d = rows;
+    int col;
+    r.divmod(within, by, col);
+    bx = panel * ph + col;
   }
 };
 

@@ -10,6 +10,7 @@
 // fragment).
 #pragma once
 #include "mma_core.hpp"
+#include "trace.hpp"
 
 namespace unit {
 
@@ -61,8 +62,13 @@ __device__ __forceinline__ void direct_load_16s(const void *sbase, u32 voff, u32
 // i receives column i of the four rows.  Two such reads make one fragment.  The chunk position inside a k row is
 // XORed with 4 * (k % 4), so that the four rows of a read fall into different bank groups (rows are 256 or 512 B).
 template <class Op, class T, int NSTAGE, class Epi, int WS, bool XOR_X, bool YT = false>
-__global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Epi::Params ep, int nk, GridMap gm) {
+__global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Epi::Params ep, int nk, GridMap gm
+                                                        UNIT_TRACE(, unsigned long long *trace_buf)) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
+  // timeline: 0 entry, 1 ring issued, 2 stage 0 landed (after the barrier), 3 last MFMA done, 4 stores issued,
+  // 5 stores acknowledged; 8 loop ticks, 9 ticks waiting for direct loads, 10 ticks in lgkmcnt + barrier, 11 entry -> loop
+  UNIT_TRACE(WaveTrace tr; tr.mark(0); const unsigned long long tk_entry = WaveTrace::ticks();
+             unsigned long long tk_a = 0, tk_b = 0, tk_c = 0, tk_vm = 0, tk_bar = 0;)
   const int t = threadIdx.x;
   const int lane = t & 63;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);  // wave-uniform: LDS positions of the direct loads stay scalar
@@ -249,13 +255,16 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
         step(kk & 1, cur, kk + 1, -1, 0, std::true_type{}, std::false_type{});
       } else {
         // stage kt+1 must have landed; stages kt+2 .. kt+NSTAGE-1 may stay in flight
+        UNIT_TRACE(tk_bar += tk_c - tk_b; tk_a = WaveTrace::ticks(); __builtin_amdgcn_sched_barrier(0);)
         if constexpr (decltype(steady)::value)
           UNIT_WAIT_VMCNT((NSTAGE - 2) * LPS);
         else
           UNIT_WAIT_VMCNT(0);
+        UNIT_TRACE(__builtin_amdgcn_sched_barrier(0); tk_b = WaveTrace::ticks(); __builtin_amdgcn_sched_barrier(0);)
         __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's reads of `cur` are done
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
+        UNIT_TRACE(tk_vm += tk_b - tk_a; tk_c = WaveTrace::ticks(); __builtin_amdgcn_sched_barrier(0);)
         // every wave has read stage kt: its buffer takes stage kt + NSTAGE
         step(kk & 1, lds + slot_next * T::STAGE, 0, kt + NSTAGE, slot, next, issue_next);
       }
@@ -268,12 +277,14 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
 #pragma unroll
   for (int s = 0; s < NSTAGE; ++s)
     if (s < nk) issue(s);
+  UNIT_TRACE(tr.mark(1);)
   // stage 0 landed?  (the NSTAGE-1 younger stages may still be in flight)
   if (nk >= NSTAGE)
     UNIT_WAIT_VMCNT((NSTAGE - 1) * LPS);
   else
     UNIT_WAIT_VMCNT(0);
   __builtin_amdgcn_s_barrier();
+  UNIT_TRACE(tr.mark(2); const unsigned long long tk_loop = WaveTrace::ticks(); tk_b = tk_c = tk_loop;)
   load_frags(lds, 0, 0);
 
   int kt = 0;
@@ -284,6 +295,9 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
   for (; kt + NSTAGE < nk; ++kt) stage(kt, kt % NSTAGE, yes{}, yes{}, yes{});
   for (; kt + 1 < nk; ++kt) stage(kt, kt % NSTAGE, no{}, no{}, yes{});
   if (kt < nk) stage(kt, kt % NSTAGE, no{}, no{}, no{});
+  UNIT_TRACE(asm volatile("s_nop 0" ::"v"(acc[T::TX - 1][T::TY - 1][15]));  // the last MFMA has written its result
+             tr.mark(3); tr.w[8] = WaveTrace::ticks() - tk_loop; tr.w[9] = tk_vm; tr.w[10] = tk_bar;
+             tr.w[11] = tk_loop - tk_entry;)
 
   if constexpr (WS == WS_Y) {
 #pragma unroll
@@ -311,6 +325,7 @@ __global__ __launch_bounds__(T::NT) void mma_dma_kernel(DmaParams p, typename Ep
   else
     Epi::template store<T>(ep, acc, wsx, wsy, x0 + wx * (T::TX * 32), y0 + wy * (T::TY * 32), lane, wave, lds,
                            gm.splits > 1, yrot);
+  UNIT_TRACE(tr.mark(4); __builtin_amdgcn_s_waitcnt(0x0F70); tr.mark(5); tr.flush(trace_buf, blockIdx.x * NW + wave);)
 }
 
 }  // namespace unit
