@@ -102,7 +102,8 @@ __device__ __forceinline__ void store_block(const typename ConvEpilogue<Op>::Par
     const int m = m0 + l32;
     int n, pix;
     p.by_ohw.divmod(m, n, pix);
-    out_t *dst = reinterpret_cast<out_t *>(p.out) + ((size_t)n * p.planar + c0 + 4 * half) * p.ohw + pix;
+    const __amdgpu_buffer_rsrc_t obuf = result_buffer(p.out);
+    const u32 dst = (u32)(n * p.planar + c0 + 4 * half) * (u32)p.ohw + (u32)pix;  // in elements
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       out4_t v = {acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]};
@@ -113,7 +114,7 @@ __device__ __forceinline__ void store_block(const typename ConvEpilogue<Op>::Par
 #pragma unroll
       for (int e = 0; e < 4; ++e)
         if (c0 + 8 * q + 4 * half + e < p.planar && m < p.npix)
-          store_result(dst + (size_t)(8 * q + e) * p.ohw, v[e]);
+          store_result(obuf, (dst + (u32)(8 * q + e) * (u32)p.ohw) * (u32)sizeof(out_t), v[e]);
     }
     return;
   }
@@ -139,7 +140,7 @@ __device__ __forceinline__ void store_block(const typename ConvEpilogue<Op>::Par
       const int c = c0 + h * 16;
       const out4_t v = *reinterpret_cast<const out4_t *>(scratch + (it * 16 + rp) * kPitch + h * 64 + piece * 16);
       if (c < p.K && m < p.npix)
-        store_result16(obuf, (obase + (u32)(c >> 4) * (u32)p.ohw * 16u) * (u32)sizeof(out_t), v);
+        store_result(obuf, (obase + (u32)(c >> 4) * (u32)p.ohw * 16u) * (u32)sizeof(out_t), v);
     }
   }
 }
@@ -202,7 +203,7 @@ __device__ __forceinline__ void store_block_q8(const typename ConvEpilogue<Op>::
   if (c < p.K && m < p.npix) {
     int n, pix;
     p.by_ohw.divmod(m, n, pix);
-    store_result16(result_buffer(p.out), (((u32)(n * (p.K >> 4)) + (u32)(c >> 4)) * (u32)p.ohw + (u32)pix) * 16u, row);
+    store_result(result_buffer(p.out), (((u32)(n * (p.K >> 4)) + (u32)(c >> 4)) * (u32)p.ohw + (u32)pix) * 16u, row);
   }
 }
 

@@ -1,6 +1,7 @@
 // Accumulator write-back for mma_kernel.  Outputs are written once and never read back by the
-// kernel, so they go out as agent-scope stores (store_result, mma_core.hpp): the lines do not stay
-// dirty in the L2 until the write-back at the end of the kernel.
+// kernel, so they go out as agent-scope non-temporal stores (store_result, mma_core.hpp): the lines
+// neither stay dirty in the L2 until the write-back at the end of the kernel nor displace the next
+// launches' operands in the memory-side cache.
 #pragma once
 #include "mma_core.hpp"
 
@@ -26,6 +27,7 @@ struct GemmEpilogue {
                                                int, char *, bool accumulate, int yrot = 0) {
     // yrot: accumulator column j (and wsy[j]) belongs to Y block (j + yrot) % TY of the wave tile
     const int l32 = lane & 31, half = lane >> 5;
+    const __amdgpu_buffer_rsrc_t cbuf = result_buffer(p.c);
 #pragma unroll
     for (int j = 0; j < T::TY; ++j) {
       const int n = yw0 + ((j + yrot) % T::TY) * 32 + l32;
@@ -42,14 +44,14 @@ struct GemmEpilogue {
             if (accumulate)
               atomicAdd(reinterpret_cast<int *>(p.c) + idx, v);
             else
-              store_result(reinterpret_cast<int *>(p.c) + idx, v);
+              store_result(cbuf, (u32)idx * 4u, v);
           } else if constexpr (OUT_F16) {
-            store_result(reinterpret_cast<_Float16 *>(p.c) + idx, (_Float16)acc[i][j][r]);  // no k-splits for f16 out
+            store_result(cbuf, (u32)idx * 2u, (_Float16)acc[i][j][r]);  // no k-splits for f16 out
           } else {
             if (accumulate)
               unsafeAtomicAdd(reinterpret_cast<float *>(p.c) + idx, acc[i][j][r]);
             else
-              store_result(reinterpret_cast<float *>(p.c) + idx, acc[i][j][r]);
+              store_result(cbuf, (u32)idx * 4u, acc[i][j][r]);
           }
         }
     }
@@ -174,7 +176,7 @@ struct ConvEpilogue {
                   unsafeAtomicAdd(dst + e, v[e]);
               }
             } else {
-              store_result16(result_buffer(p.out), (u32)((obase[it] + (size_t)(c >> 4) * p.ohw * 16) * sizeof(out_t)), v);
+              store_result(result_buffer(p.out), (u32)((obase[it] + (size_t)(c >> 4) * p.ohw * 16) * sizeof(out_t)), v);
             }
           }
         }

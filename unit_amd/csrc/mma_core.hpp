@@ -28,31 +28,30 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef unsigned int u32;
 
-// Result stores.  Results are written once and never read back by the kernel that writes them, so they are stored at
-// agent scope (sc1): the line goes through the XCD's L2 to memory at once instead of waiting there, dirty, for the
-// write-back at the end of the kernel.  Measured on a 102.8 MB fill: 15.05 us (6.83 TB/s) against 16.44 us for plain
-// stores and 16.56 us for non-temporal ones; sc0 changes nothing, nt on top of sc1 loses half of the gain.
-// Scalars go out as relaxed agent-scope atomic stores (global_store_dword / _short ... sc1); 16-byte vectors as raw
-// buffer stores with the sc1 policy bit, at a 32-bit byte offset from the tensor's base (tensors stay below 2^31
-// bytes).  Both are instructions the compiler knows, so its hazard and wait-count passes see them.
+// Result stores.  Results are written once and never read back by the kernel that writes them, so they go out as
+// agent-scope, non-temporal stores (sc1 nt): sc1 sends the line through the XCD's L2 to memory at once instead of
+// leaving it there, dirty, for the write-back at the end of the kernel; nt keeps it from displacing the operands of
+// the launches that follow in the memory-side cache.  Measured, 102.8 MB of results: a plain fill 16.4 us on a
+// destination that the cache still holds / 17.3 us on a cold one, nt 16.6 / 16.7, sc1 15.1 / 16.0, sc1 nt 15.6 / 15.8;
+// the ResNet-50 batch-32 convolution step 0.5415 ms with nt, 0.5777 ms with sc1 alone (its launches find their
+// operands evicted: the layers on cold operands take 651 us against 591 us), 0.5324 ms with sc1 nt.
+// They are raw buffer stores at a 32-bit byte offset from the tensor's base (tensors stay below 2^31 bytes), the
+// form that takes the policy bits as an operand the compiler knows: its hazard and wait-count passes see the stores
+// (written as inline assembly they were followed by a write of the data registers inside the store's hazard window).
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+constexpr int kResultPolicy = 16 | 2;  // sc1 | nt
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t result_buffer(void *base) {
   return __builtin_amdgcn_make_buffer_rsrc(base, 0, -1, 0x00020000);
 }
 template <class V>
-__device__ __forceinline__ void store_result16(__amdgpu_buffer_rsrc_t buf, u32 byte_offset, V v) {
-  static_assert(sizeof(V) == 16, "a 16-byte vector");
-  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), buf, (int)byte_offset, 0, 16 /* sc1 */);
-}
-__device__ __forceinline__ void store_result(int *p, int v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void store_result(float *p, float v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void store_result(_Float16 *p, _Float16 v) {
-  __hip_atomic_store(reinterpret_cast<unsigned short *>(p), __builtin_bit_cast(unsigned short, v), __ATOMIC_RELAXED,
-                     __HIP_MEMORY_SCOPE_AGENT);
+__device__ __forceinline__ void store_result(__amdgpu_buffer_rsrc_t buf, u32 byte_offset, V v) {
+  static_assert(sizeof(V) == 16 || sizeof(V) == 4 || sizeof(V) == 2, "results are stored 16, 4 or 2 bytes at a time");
+  if constexpr (sizeof(V) == 16)
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), buf, (int)byte_offset, 0, kResultPolicy);
+  else if constexpr (sizeof(V) == 4)
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned int, v), buf, (int)byte_offset, 0, kResultPolicy);
+  else
+    __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, v), buf, (int)byte_offset, 0, kResultPolicy);
 }
 
 // 4-byte-aligned views for gathers whose address is only dword aligned
