@@ -328,6 +328,27 @@ REQUANT_CASES = [
 ]
 
 
+def test_conv2d_fp16_prepared_large_window_keeps_direct_kernels(dev, oracle, monkeypatch):
+    """A 7 x 7 window has 49 positions, more than the 32-bit position set of the LDS-shared kernels holds: whatever
+    variant is forced, the prepared fp16 convolution runs a direct kernel, and integer-valued data reproduces the
+    float64 reference bit for bit."""
+    from unit_amd import _lib
+    N, C, H, W, K, ks = 1, 16, 12, 13, 32, 7
+    a = (rng.uniform_u8((N, C // 16, H, W, 16), 61) % 7).astype(np.float16) - 3
+    b = (rng.uniform_u8((K // 16, C // 16, ks, ks, 16, 16), 62) % 5).astype(np.float16) - 2
+    ref = oracle.conv2d_nchw16c_f16(a, b, 1, 1)
+    ta, p = _t(a, dev), U.prepare_conv2d_weight(_t(b, dev))
+    L = _lib.load()
+    for v in range(1, L.unit_conv_variant_count() + 1):
+        if L.unit_conv_variant_is_direct(v - 1) != 2:
+            continue
+        monkeypatch.setenv("UNIT_AMD_CONV_VARIANT", str(v))
+        out = U.conv2d_NCHW16c_OHWI16o(ta, p, 1, 1)
+        torch.cuda.synchronize()
+        assert U.last_variant().startswith("f16prep"), (v, U.last_variant())
+        assert np.array_equal(out.cpu().numpy().astype(np.float64), ref), (v, U.last_variant())
+
+
 @pytest.mark.parametrize("N,C,H,W,K,ks,stride,pad,scale,shift,with_bias", REQUANT_CASES)
 def test_conv2d_requant_u8(dev, oracle, N, C, H, W, K, ks, stride, pad, scale, shift, with_bias):
     """Requantised u8 output against the oracle's integer definition (bit-exact), on inputs scaled so that the

@@ -58,3 +58,47 @@ def test_static_scratch_gemm_without_k_splits_and_beyond_its_limit(dev):
     c = torch.zeros((M, N), dtype=torch.float32, device=dev)
     rc = L.unit_gemm_f16_static(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, 0, torch.cuda.current_stream().cuda_stream)
     assert rc == -1 and b"static buffer holds" in L.unit_last_error()
+
+
+def test_static_scratch_gemm_allocates_nothing_and_replays_in_a_graph(dev):
+    """The property the entry point is for: after one call outside capture (it resolves the scratch array's address
+    on this device), a k-split call and a call without k-splits are captured into one HIP graph; every replay --
+    with eager launches and synchronisations between them -- reproduces the eager results bit for bit, and the free
+    device memory is the same before and after the calls."""
+    L = _lib.load()
+    shapes = ((128, 768, 3072), (512, 512, 256))  # 21 k-splits through the scratch array; 16 tiles, no split
+    ops = []
+    for i, (M, N, K) in enumerate(shapes):
+        a = torch.from_numpy(rng.normal_f16((M, K), 41 + i, 1.0 / np.sqrt(K))).to(dev)
+        b = torch.from_numpy(rng.normal_f16((K, N), 51 + i)).to(dev)
+        ops.append((a, b, torch.empty((M, N), dtype=torch.float32, device=dev), M, N, K))
+
+    def run(stream):
+        for a, b, c, M, N, K in ops:
+            _lib.check(L.unit_gemm_f16_static(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, 0, stream))
+
+    run(torch.cuda.current_stream().cuda_stream)  # outside capture: symbol address, kernel attributes
+    torch.cuda.synchronize()
+    eager = [c.clone() for _, _, c, _, _, _ in ops]
+    free_before = torch.cuda.mem_get_info()[0]
+    run(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run(torch.cuda.current_stream().cuda_stream)
+    for replay in range(3):
+        for _, _, c, _, _, _ in ops:
+            c.fill_(float(replay) - 7.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for want, (_, _, c, _, _, _) in zip(eager, ops):
+            assert torch.equal(want, c), replay
+        # eager work of the same entry point between replays: the shared scratch array is rewritten
+        a, b, c, M, N, K = ops[0]
+        other = torch.empty_like(c)
+        _lib.check(L.unit_gemm_f16_static(a.data_ptr(), b.data_ptr(), other.data_ptr(), M, N, K, 0,
+                                          torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        assert torch.equal(other, eager[0])

@@ -59,6 +59,8 @@ struct LdsShape {
 // them (it would make LDS reads that follow a direct load wait for all of them); the kernel's own vmcnt waits
 // order them.  Weight fragments: scalar base + the lane's 16-byte offset.  Pixel rows: a raw buffer load, whose
 // out-of-range lanes store zeros into LDS -- the hardware's own zero padding.
+// The statements write m0 without naming it as a clobber: the compiler reserves m0 (it sets it right before each
+// instruction of its own that reads it and keeps no value in it across statements) and rejects it in a clobber list.
 __device__ __forceinline__ void dma_global_16(u32 lds_addr, u32 voff, const void *sbase) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
 }

@@ -130,7 +130,9 @@ const TunedConv kTunedF16Prepared[] = {
 // lds_ok: the entry point also has the LDS-shared kernels (int8, 16-channel blocks).
 ConvPlan plan_prepared(const unit_conv_desc *d, const ConvGeom &g, int kbytes, const TunedConv *table, int ntable,
                        bool int8, bool lds_ok = false) {
-  lds_ok = lds_ok && d->cb == 16;
+  // the LDS-shared kernels keep a window's positions as a 32-bit set: larger windows (possible for fp16, whose direct
+  // kernels have no such limit) stay on the direct kernels, whatever a table row or an override names
+  lds_ok = lds_ok && d->cb == 16 && d->KH * d->KW <= 31;
   ConvPlan p = plan_conv(d, g.npix, kbytes, table, ntable, int8, true, false, lds_ok);
   const TileShape &t = kConvTiles[p.variant];
   if (!(t.direct || (t.lds && lds_ok))) p = heuristic_plan(g.npix, d->K, kbytes, int8, true, d->sh * d->sw > 1);

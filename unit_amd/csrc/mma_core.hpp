@@ -34,7 +34,8 @@ typedef unsigned int u32;
 // the launches that follow in the memory-side cache.  Measured, 102.8 MB of results: a plain fill 16.4 us on a
 // destination that the cache still holds / 17.3 us on a cold one, nt 16.6 / 16.7, sc1 15.1 / 16.0, sc1 nt 15.6 / 15.8;
 // the ResNet-50 batch-32 convolution step 0.5415 ms with nt, 0.5777 ms with sc1 alone (its launches find their
-// operands evicted: the layers on cold operands take 651 us against 591 us), 0.5324 ms with sc1 nt.
+// operands evicted: the layers on cold operands take 651 us against 591 us), 0.5324 ms with sc1 nt; the chain of 52
+// requantising layers, each reading the previous one's u8 result, 497 us with sc1 nt against 513 us with sc1.
 // They are raw buffer stores at a 32-bit byte offset from the tensor's base (tensors stay below 2^31 bytes), the
 // form that takes the policy bits as an operand the compiler knows: its hazard and wait-count passes see the stores
 // (written as inline assembly they were followed by a write of the data registers inside the store's hazard window).
@@ -43,15 +44,15 @@ constexpr int kResultPolicy = 16 | 2;  // sc1 | nt
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t result_buffer(void *base) {
   return __builtin_amdgcn_make_buffer_rsrc(base, 0, -1, 0x00020000);
 }
-template <class V>
+template <int POLICY = kResultPolicy, class V>
 __device__ __forceinline__ void store_result(__amdgpu_buffer_rsrc_t buf, u32 byte_offset, V v) {
   static_assert(sizeof(V) == 16 || sizeof(V) == 4 || sizeof(V) == 2, "results are stored 16, 4 or 2 bytes at a time");
   if constexpr (sizeof(V) == 16)
-    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), buf, (int)byte_offset, 0, kResultPolicy);
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), buf, (int)byte_offset, 0, POLICY);
   else if constexpr (sizeof(V) == 4)
-    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned int, v), buf, (int)byte_offset, 0, kResultPolicy);
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned int, v), buf, (int)byte_offset, 0, POLICY);
   else
-    __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, v), buf, (int)byte_offset, 0, kResultPolicy);
+    __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, v), buf, (int)byte_offset, 0, POLICY);
 }
 
 // 4-byte-aligned views for gathers whose address is only dword aligned
