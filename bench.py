@@ -77,6 +77,9 @@ def main():
                     help="launch one kernel 20 times and exit (for rocprofv3): a ResNet-50 layer name such as "
                          "3x3_256_256@14 (append :f16 for the fp16 convolution, :cold to cycle operand copies), "
                          "or gemm_i8 / gemm_i8_prepared / gemm_f16 / gemm_f16_prepared / gemm_f16_2048 / copy / pack_u8")
+    ap.add_argument("--profile-launches", type=int, default=20, metavar="N",
+                    help="launches of the --profile kernel (default 20; the 4096^3 GEMMs reach their steady-state clocks "
+                         "after ~300 launches: profile 500 and read the last ones)")
     ap.add_argument("--profile-batch", type=int, default=None, metavar="N",
                     help="batch of the --profile launches of a layer (default: the benchmark's 32)")
     args = ap.parse_args()
@@ -113,8 +116,8 @@ def main():
         """Mean launch-to-launch time of `iters` back-to-back launches (HIP events on the launch stream); with
         bursts > 1 the median burst -- one protocol for every leg.  The fastest burst is left in last_min[0].
         `warm` untimed launches come first: the clocks of this part follow the load of whatever ran just before
-        (a 4096^3 GEMM takes ~10 % longer in the first milliseconds after an idle phase), so the GEMM legs warm up
-        with sustained launches and report the steady state."""
+        (launch by launch a 4096^3 GEMM runs 58, 70 around the 50th, then 57 us from the ~300th launch on), so the GEMM
+        legs warm up with sustained launches and report the steady state."""
         for _ in range(warm):
             fn()
         torch.cuda.synchronize()
@@ -156,10 +159,10 @@ def main():
             a = torch.empty(1 << 30, dtype=torch.uint8, device=dev)   # point for FETCH_SIZE / WRITE_SIZE
             b = torch.empty_like(a)
             fn = lambda: b.copy_(a)
-        for _ in range(20):
+        for _ in range(args.profile_launches):
             fn()
         torch.cuda.synchronize()
-        print(json.dumps({"profiled": prof, "launches": 20, "kernel": U.last_variant()}))
+        print(json.dumps({"profiled": prof, "launches": args.profile_launches, "kernel": U.last_variant()}))
         return
 
     def cold_copies(tensors, per_bytes):
@@ -368,7 +371,8 @@ def main():
     g_rm = lambda: _lib.check(L.unit_dense_u8s8s32(a8.data_ptr(), w8.data_ptr(), c8.data_ptr(), M, N, K, stream))
     g_pk = lambda: _lib.check(L.unit_dense_dotprod_u8s8s32(a8.data_ptr(), wp8.data_ptr(), c8.data_ptr(), M, N, K,
                                                             stream))
-    GEMM_WARM = 100  # sustained launches before the timed bursts (7-13 ms)
+    GEMM_WARM = 400  # sustained launches before the timed bursts (25-50 ms): a 4096^3 GEMM starts at boost clocks,
+    # is throttled ~15 % around its 50th launch and settles only after ~300 launches
     us_rm = time_us(g_rm, 30, warm=GEMM_WARM, bursts=3)
     v_rm, min_rm = U.last_variant(), last_min[0]
     us_pk = time_us(g_pk, 30, warm=GEMM_WARM, bursts=3)

@@ -172,14 +172,17 @@ def test_bench_final_line_fits_the_tail_budget():
         "gemm_int8_us": 80.39, "gemm_int8_pct_peak": 33.97, "gemm_int8_prepared_w_us": 72.31, "gemm_int8_prepared_w_pct_peak": 37.77, "gemm_fp16_us": 143.58, "gemm_fp16_tflops": 957.2,
         "gemm_fp16_pct_peak": 38.05, "gemm_fp16_prepared_b_us": 119.64, "gemm_fp16_prepared_b_pct_peak": 45.66,
         "gemm_fp16_max_rel_err": 0.000247, "sum_layers_cold_us": 612.3, "launch": "hipgraph",
+        "roofline_step": dict(ideal_us=217.2, frac=0.377, bytes=1702945984, ops=246779215872, launches=53),
         "fp16_conv": dict(stack_us=618.2, tflops=387.0),
-        "probe": {"int8_tops": 4409.7, "fp16_tflops": 2327.2, "int8_tops_random_operands": 3374.3,
-                  "fp16_tflops_random_operands": 1646.7},
+        "gemm_int8_frac_of_probe": 0.565, "gemm_fp16_frac_of_probe": 0.737,
+        "probe": {"int8_tops": 4409.7, "fp16_tflops": 2327.2, "int8_tops_bench_operands": 3374.3,
+                  "fp16_tflops_bench_operands": 1646.7},
     }
     s = bench.compact_line(dict(line))
     assert len(s) <= bench.FINAL_LINE_BUDGET and "\n" not in s
     back = json.loads(s)
-    for key in ("metric", "value", "unit", "ms_per_step", "roofline", "cpu_baseline", "config"):
+    for key in ("metric", "value", "unit", "ms_per_step", "roofline", "roofline_step", "cpu_baseline", "config",
+                "gemm_int8_frac_of_probe", "gemm_fp16_frac_of_probe"):
         assert key in back
     # an oversized line sheds optional keys, never the contract's
     line["probe"] = {f"k{i}": "x" * 40 for i in range(40)}
@@ -189,13 +192,21 @@ def test_bench_final_line_fits_the_tail_budget():
 
 def test_bench_traffic_table_names_its_profiles():
     import os
+    import re
 
     import bench
     table = bench.read_traffic_table()
     assert table, "profiles/hbm_traffic_table.txt is missing or empty"
+    root = os.path.dirname(bench.__file__)
+    tuned = open(os.path.join(root, "unit_amd", "csrc", "tuned_conv_i8_prepared.inc")).read()
     for (layer, kernel), (nbytes, src) in table.items():
         assert any(s.name == layer for s in WL.RESNET50) and nbytes > 0
-        assert os.path.exists(os.path.join(os.path.dirname(bench.__file__), src)), src
+        assert os.path.exists(os.path.join(root, src)), src
+        # the row describes the kernel variant that the tuned table picks for this layer at batch 32 (the benchmark's
+        # launch), and the profile it points to was taken on that variant: otherwise bench.py would report no traffic
+        m = re.search(r"resnet50 b32 " + re.escape(layer) + r": [0-9.]+ us \(([^)]*)\)", tuned)
+        assert m and m.group(1) == kernel, (layer, kernel, m and m.group(1))
+        assert f"unit_last_variant(): {kernel}" in open(os.path.join(root, src)).read(), src
 
 
 def test_padding_bound_is_checked_on_the_host():

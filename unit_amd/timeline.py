@@ -79,8 +79,8 @@ def main(argv):
                 bop = U.prepare_gemm_b(b) if what.endswith("prepared") else b
                 fn = lambda: U.gemm_fp16(a, bop)
                 ideal_ticks = (2 * n // 32) * 8 * 32 * 2
-            us = timed(fn, 150)
-            points, warm = GEMM_POINTS, 150
+            us = timed(fn, 400)  # the clocks settle after ~300 sustained launches
+            points = GEMM_POINTS
         else:
             match = [s for s in WL.RESNET50 if s.name == what and s.C % 16 == 0]
             if not match:
