@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), f"libunit_amd.so does not export {n}"
     assert sorted(_lib.SYMBOLS) == names, "unit_amd/_lib.py and include/unit_amd.h disagree"
-    assert lib.unit_version() == 105
+    assert lib.unit_version() == 106
 
 
 def test_conv_desc_matches_the_header_struct():

@@ -203,7 +203,7 @@ extern "C" int unit_trace_words(void) { return unit::kTraceWords; }
 extern "C" int unit_trace_waves(void) { return unit::kTraceWaves; }
 #endif
 
-extern "C" int unit_version(void) { return 105; }  // 1.5: fp16 GEMM k-splits through a workspace or the library's static scratch; 1.4: LDS-shared convolution variants (16 KiB of zeros behind prepared int8 weights), dense on a prepared weight
+extern "C" int unit_version(void) { return 106; }  // 1.6: results stored sc1 nt, row-major int8 dense on the direct-to-LDS kernel, unit_mfma_peak mode 5 (the fp16 benchmark's operand distribution); 1.5: fp16 GEMM k-splits through a workspace or the library's static scratch; 1.4: LDS-shared convolution variants (16 KiB of zeros behind prepared int8 weights), dense on a prepared weight
 
 extern "C" const char *unit_last_error(void) { return unit::error_buf(); }
 
