@@ -116,8 +116,8 @@ def main():
         """Mean launch-to-launch time of `iters` back-to-back launches (HIP events on the launch stream); with
         bursts > 1 the median burst -- one protocol for every leg.  The fastest burst is left in last_min[0].
         `warm` untimed launches come first: the clocks of this part follow the load of whatever ran just before
-        (launch by launch a 4096^3 GEMM runs 58, 70 around the 50th, then 57 us from the ~300th launch on), so the GEMM
-        legs warm up with sustained launches and report the steady state."""
+        (launch by launch the 4096^3 int8 GEMM runs 69, 82 around the 50th, then 65 us from the ~300th launch on), so the
+        GEMM legs warm up with sustained launches and report the steady state."""
         for _ in range(warm):
             fn()
         torch.cuda.synchronize()
