@@ -95,6 +95,9 @@ int conv_geom(const unit_conv_desc *d, int tapb, ConvGeom *g, const char *what) 
   g->nopad = !(d->pt || d->pl || d->pb || d->pr);
   g->by_plane = g->by_ohw;
   g->by_kd = FastDiv::make(1);
+  g->row_ones = 0;
+  if (d->dh == 1 && d->dw == 1 && d->KH * d->KW <= 31)
+    for (int kh = 0; kh < d->KH; ++kh) g->row_ones |= 1u << (kh * d->KW);
   return UNIT_OK;
 }
 

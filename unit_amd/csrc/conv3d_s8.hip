@@ -62,6 +62,7 @@ extern "C" int unit_conv3d_ncdhwc_s8s8s32(const unit_conv3d_desc *d, const void 
   g.D = d->D; g.KD = d->KD; g.sd = d->stride; g.nopad = 1;
   g.by_plane = FastDiv::make(OH * OW);
   g.by_kd = FastDiv::make(d->KD);
+  g.row_ones = 0;  // no padding: no window positions to mask
   // the launcher only reads K from the 2-D descriptor; the planner keys on pixels, channels and reduction length
   unit_conv_desc d2{d->N, d->C, d->H, d->W, d->K, d->KH, d->KW, d->stride, d->stride, 0, 0, 0, 0, 1, 1, cb};
   ConvPlan p = plan_conv(&d2, g.npix, g.ntaps * cb, nullptr, 0, true, true);

@@ -213,11 +213,12 @@ __global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !
                                                      UNIT_TRACE(, unsigned long long *trace_buf)) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   constexpr int TX = S::TX, TY = S::TY, KG = S::KG, D = S::D;
-  // timeline: 0 entry, 1 arguments fetched, 2 tables and per-lane window state built, 3 past the barrier, 4 ring
-  // issued, 5 reduction done (accumulators complete), 6 k-groups summed, 7 stores issued and acknowledged
+  // timeline: 0 entry, 1 arguments fetched, 2 the ring's weight loads issued, 3 per-lane window state built, 4 the
+  // ring's pixel loads issued, 5 reduction done (accumulators complete), 6 k-groups summed, 7 stores issued and
+  // acknowledged
   UNIT_TRACE(WaveTrace tr; tr.mark(0);)
   {
-    // Touch every 64-byte line of the 260 bytes of kernel arguments at once: the compiler fetches the arguments
+    // Touch each of the five 64-byte lines of kernel arguments at once: the compiler fetches the arguments
     // where it first needs them, in three dependent rounds of scalar loads before the first operand fetch.
     const auto *ka = (const __attribute__((address_space(4))) int *)__builtin_amdgcn_kernarg_segment_ptr();
     const int w0 = ka[0], w1 = ka[16], w2 = ka[32], w3 = ka[48], w4 = ka[64];
@@ -248,7 +249,7 @@ __global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !
   // C4: a k-step is (channel block, kh); the table holds the row's offset for both halves and kh
   const int nsteps = C4 ? g.c4_steps : (kInt ? (g.ntaps + 1) >> 1 : g.ntaps);
   const int ntab = kInt ? 2 * nsteps : nsteps;
-  for (int e = threadIdx.x; e < ntab; e += S::NT) {
+  auto tap_entry = [&](int e) __attribute__((always_inline)) {
     v2i ent = {0, 31};
     if constexpr (C4) {
       int rest, kh, ci, kd;
@@ -264,13 +265,14 @@ __global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !
       ent[0] = (((ci * g.D + kd) * g.H + kh * g.dh) * g.W + kw * g.dw) * TAPB;
       ent[1] = g.nopad ? 0 : kh * g.KW + kw;
     }
-    tab[e] = ent;
-  }
-  if constexpr (KG > 1 && !kParked) {
-    v4i *z = reinterpret_cast<v4i *>(tiles);
-    for (int e = threadIdx.x; e < (S::TILE + S::WSUM) / 16; e += S::NT) z[e] = v4i{0, 0, 0, 0};
-  }
+    return ent;
+  };
 
+  // The prologue is ordered by what the first loads need, because a wave's life at batch 32 is a chain of
+  // latencies rather than a rate: the ring's weight fragments depend on the workgroup's place alone and go out
+  // first; the ring's pixel fragments need this lane's window origin and the ring's own tap entries, which lane q
+  // computes for tap q of the ring and the wave reads back lane by lane; the tap table in LDS, the zeroed sums and the
+  // barrier that publishes them are only needed by the fetches after the ring and follow the loads.
   int bx, by, split;
   gm.locate(blockIdx.x, bx, by, split);
   const int x0 = bx * S::BX, y0 = by * S::BY;
@@ -296,20 +298,67 @@ __global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !
 #pragma unroll
     for (int e = 0; e < 4; ++e) wtap[e] = (u32)min(4 * half + e, g.KW - 1) * 64u;
   }
-  // per-channel addend read from memory (bias; with PREP and u8 data the shift correction): one
-  // wave contributes it, and the load is issued here so that its latency hides behind the loop
-  int addv[TX];
+  auto for_slots = [&](auto f) __attribute__((always_inline)) {
+    f(std::integral_constant<int, 0>{});
+    f(std::integral_constant<int, 1>{});
+    if constexpr (D > 2) f(std::integral_constant<int, 2>{});
+    if constexpr (D > 3) f(std::integral_constant<int, 3>{});
+    if constexpr (D > 4) f(std::integral_constant<int, 4>{});
+    if constexpr (D > 5) f(std::integral_constant<int, 5>{});
+    if constexpr (D > 6) f(std::integral_constant<int, 6>{});
+    if constexpr (D > 7) f(std::integral_constant<int, 7>{});
+  };
+
+  // prefetch ring: D k-steps of fragments in registers
+  v4i xf[D][TX], yf[D][TY];
+  int ym[S::PAD && !C4 ? D : 1][TY];  // all ones where the tap lies inside the image, else 0
+  v4i ym4[C4 ? D : 1][TY];           // C4: the same per tap of the fragment
+  const u32 last_tap_off = (u32)(g.ntaps - 1) * (u32)WTAP;
+
+  // this wave's k-steps [s0, s1); fetches past the last one re-read it
+  const int s0 = nsteps * wave / KG, s1 = nsteps * (wave + 1) / KG;
+  const int slast = s1 - 1;
+
+  // Offsets are unsigned 32-bit values added to a uniform base pointer, so a load needs no 64-bit
+  // address arithmetic per lane.
+  // The weight fragments of k-step `scur`.
+  auto fetch_w = [&](auto slot, int scur) __attribute__((always_inline)) {
+    constexpr int U = decltype(slot)::value;
+    const int t = kInt ? 2 * scur + half : scur;
+    const u32 xs = (u32)scur * 1024u;  // PREP: a k-step of a 32-channel block is 1 KiB
+    // int8: the odd tap past the end re-reads the last tap's weights.  Its data is staged as
+    // zero padding, and a padded position contributes -128 * w to the accumulator and +128 * w
+    // through the weight-sum correction (SHIFT) or 0 * w (signed data), whatever w is.
+    u32 xk = (u32)t * (u32)WTAP;
+    xk = xk < last_tap_off ? xk : last_tap_off;
 #pragma unroll
-  for (int i = 0; i < TX; ++i) {
-    addv[i] = 0;
-    if constexpr (kInt) {
-      const int c = x0 + i * 32 + l32;
-      if (ep.bias != nullptr && wave == 0 && c < ep.K) addv[i] = ep.bias[c];
-      if constexpr (Q8) {
-        if (ep.bias2 != nullptr && wave == 0 && c < ep.K) addv[i] += ep.bias2[c];
+    for (int i = 0; i < TX; ++i) {
+      const u32 o = xoff[i] + xk;
+      if constexpr (PREP) {
+        xf[U][i] = *reinterpret_cast<const v4i *>(wgt + xoff[i] + xs);
+      } else if constexpr (C4) {
+        const u32 xr = (u32)scur * (u32)(g.KW * 64);  // this k-step's window row
+#pragma unroll
+        for (int d = 0; d < 4; ++d) xf[U][i][d] = *reinterpret_cast<const int *>(wgt + xoff[i] + xr + wtap[d]);
+      } else if constexpr (kInt) {
+#pragma unroll
+        for (int d = 0; d < 4; ++d) xf[U][i][d] = *reinterpret_cast<const int *>(wgt + o + d * 64);
+      } else {
+        v8h h;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) h[k] = *reinterpret_cast<const _Float16 *>(wgt + o + k * 32);
+        xf[U][i] = __builtin_bit_cast(v4i, h);
       }
     }
+  };
+  if (s0 < s1) {
+    for_slots([&](auto u) __attribute__((always_inline)) {
+      fetch_w(u, min(s0 + decltype(u)::value, slast));
+    });
   }
+  __builtin_amdgcn_sched_barrier(0);
+  UNIT_TRACE(tr.mark(2);)
+
   // data: byte offset of the window origin of this lane's pixel per 32-pixel block, and the set of
   // window positions (kh, kw) that fall inside the image (none for lanes past the last pixel)
   int pixoff[TY];
@@ -339,70 +388,25 @@ __global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !
         }
       } else if constexpr (S::PAD) {
         u32 cols = 0, bits = 0;  // columns kw inside the image; then one copy of them per row kh inside
-        for (int kw = 0; kw < g.KW; ++kw) cols |= (u32)((u32)(iw0 + kw * g.dw) < (u32)g.W) << kw;
-        for (int kh = 0; kh < g.KH; ++kh)
-          if ((u32)(ih0 + kh * g.dh) < (u32)g.H) bits |= cols << (kh * g.KW);
+        if (g.row_ones) {  // undilated: columns [ka, kb) and rows [ra, rb) of the window are inside
+          const int ka = min(max(-iw0, 0), g.KW), kb = min(max(g.W - iw0, ka), g.KW);
+          const int ra = min(max(-ih0, 0), g.KH), rb = min(max(g.H - ih0, ra), g.KH);
+          cols = (1u << kb) - (1u << ka);
+          bits = cols * (g.row_ones & ((1u << (rb * g.KW)) - (1u << (ra * g.KW))));
+        } else {
+          for (int kw = 0; kw < g.KW; ++kw) cols |= (u32)((u32)(iw0 + kw * g.dw) < (u32)g.W) << kw;
+          for (int kh = 0; kh < g.KH; ++kh)
+            if ((u32)(ih0 + kh * g.dh) < (u32)g.H) bits |= cols << (kh * g.KW);
+        }
         inside[j] = g.nopad ? 1u : bits;  // without padding every real tap carries position 0
       }
     }
   }
+  UNIT_TRACE(asm volatile("s_nop 0" ::"v"(pixoff[0]), "v"(inside[0])); tr.mark(3);)
 
-  typename Op::acc_t acc[TX][TY];
-#pragma unroll
-  for (int i = 0; i < TX; ++i)
-#pragma unroll
-    for (int j = 0; j < TY; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-  int wsx[TX];
-#pragma unroll
-  for (int i = 0; i < TX; ++i) wsx[i] = 0;
-
-  // prefetch ring: D k-steps of fragments in registers
-  v4i xf[D][TX], yf[D][TY];
-  int ym[S::PAD && !C4 ? D : 1][TY];  // all ones where the tap lies inside the image, else 0
-  v4i ym4[C4 ? D : 1][TY];           // C4: the same per tap of the fragment
-  const u32 last_tap_off = (u32)(g.ntaps - 1) * (u32)WTAP;
-
-  // Fetches run through the k-steps in order; `sf` is the next one (it stops at the wave's last
-  // k-step, so surplus fetches re-read that one) and `ecur` its tap table entry, read one fetch
-  // ahead so that the LDS latency is not in the way of the loads.
-  // Offsets are unsigned 32-bit values added to a uniform base pointer, so a load needs no 64-bit
-  // address arithmetic per lane.
-  int sf = 0, slast = 0;
-  v2i ecur = {0, 31};
-  auto fetch = [&](auto slot) __attribute__((always_inline)) {
+  // The pixel fragments of one k-step, whose tap table entry for this lane's half is `e`.
+  auto fetch_d = [&](auto slot, v2i e) __attribute__((always_inline)) {
     constexpr int U = decltype(slot)::value;
-    const int t = kInt ? 2 * sf + half : sf;
-    const int scur = sf;
-    const u32 xs = (u32)scur * 1024u;  // PREP: a k-step of a 32-channel block is 1 KiB
-    const v2i e = ecur;
-    sf = sf < slast ? sf + 1 : slast;
-    ecur = tab[kInt ? 2 * sf + half : sf];
-    // int8: the odd tap past the end re-reads the last tap's weights.  Its data is staged as
-    // zero padding, and a padded position contributes -128 * w to the accumulator and +128 * w
-    // through the weight-sum correction (SHIFT) or 0 * w (signed data), whatever w is.
-    u32 xk = (u32)t * (u32)WTAP;
-    xk = xk < last_tap_off ? xk : last_tap_off;
-#pragma unroll
-    for (int i = 0; i < TX; ++i) {
-      const u32 o = xoff[i] + xk;
-      if constexpr (PREP) {
-        xf[U][i] = *reinterpret_cast<const v4i *>(wgt + xoff[i] + xs);
-      } else if constexpr (C4) {
-        const u32 xr = (u32)scur * (u32)(g.KW * 64);  // this k-step's window row
-#pragma unroll
-        for (int d = 0; d < 4; ++d) xf[U][i][d] = *reinterpret_cast<const int *>(wgt + xoff[i] + xr + wtap[d]);
-      } else if constexpr (kInt) {
-#pragma unroll
-        for (int d = 0; d < 4; ++d) xf[U][i][d] = *reinterpret_cast<const int *>(wgt + o + d * 64);
-      } else {
-        v8h h;
-#pragma unroll
-        for (int k = 0; k < 8; ++k) h[k] = *reinterpret_cast<const _Float16 *>(wgt + o + k * 32);
-        xf[U][i] = __builtin_bit_cast(v4i, h);
-      }
-    }
 #pragma unroll
     for (int j = 0; j < TY; ++j) {
       if constexpr (C4) {
@@ -424,6 +428,71 @@ __global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !
         yf[U][j] = *reinterpret_cast<const v4i *>(data + (u32)(pixoff[j] + e[0]));
       }
     }
+  };
+  if (s0 < s1) {
+    // lane q holds the entry of the ring's tap q (int8: two taps per k-step, one per half of the wave)
+    const int e0 = kInt ? 2 * s0 : s0;
+    const v2i mine = e0 + lane < ntab ? tap_entry(e0 + lane) : v2i{0, 31};
+    for_slots([&](auto u) __attribute__((always_inline)) {
+      const int q = min((int)decltype(u)::value, slast - s0);  // uniform
+      v2i e;
+      if constexpr (kInt) {
+        const int a0 = __builtin_amdgcn_readlane(mine[0], 2 * q), a1 = __builtin_amdgcn_readlane(mine[1], 2 * q);
+        const int b0 = __builtin_amdgcn_readlane(mine[0], 2 * q + 1), b1 = __builtin_amdgcn_readlane(mine[1], 2 * q + 1);
+        e = half ? v2i{b0, b1} : v2i{a0, a1};
+      } else {
+        e = v2i{__builtin_amdgcn_readlane(mine[0], q), __builtin_amdgcn_readlane(mine[1], q)};
+      }
+      fetch_d(u, e);
+    });
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  UNIT_TRACE(tr.mark(4);)
+
+  // per-channel addend read from memory (bias; with PREP and u8 data the shift correction): one
+  // wave contributes it, and the load is issued here so that its latency hides behind the loop
+  int addv[TX];
+#pragma unroll
+  for (int i = 0; i < TX; ++i) {
+    addv[i] = 0;
+    if constexpr (kInt) {
+      const int c = x0 + i * 32 + l32;
+      if (ep.bias != nullptr && wave == 0 && c < ep.K) addv[i] = ep.bias[c];
+      if constexpr (Q8) {
+        if (ep.bias2 != nullptr && wave == 0 && c < ep.K) addv[i] += ep.bias2[c];
+      }
+    }
+  }
+  // the tap table for the fetches after the ring, and the zeroed sums
+  for (int e = threadIdx.x; e < ntab; e += S::NT) tab[e] = tap_entry(e);
+  if constexpr (KG > 1 && !kParked) {
+    v4i *z = reinterpret_cast<v4i *>(tiles);
+    for (int e = threadIdx.x; e < (S::TILE + S::WSUM) / 16; e += S::NT) z[e] = v4i{0, 0, 0, 0};
+  }
+
+  typename Op::acc_t acc[TX][TY];
+#pragma unroll
+  for (int i = 0; i < TX; ++i)
+#pragma unroll
+    for (int j = 0; j < TY; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+  int wsx[TX];
+#pragma unroll
+  for (int i = 0; i < TX; ++i) wsx[i] = 0;
+
+  // Fetches after the ring run through the k-steps in order; `sf` is the next one (it stops at the wave's last
+  // k-step, so surplus fetches re-read that one) and `ecur` its tap table entry, read one fetch
+  // ahead so that the LDS latency is not in the way of the loads.
+  int sf = 0;
+  v2i ecur = {0, 31};
+  auto fetch = [&](auto slot) __attribute__((always_inline)) {
+    const int scur = sf;
+    const v2i e = ecur;
+    sf = sf < slast ? sf + 1 : slast;
+    ecur = tab[kInt ? 2 * sf + half : sf];
+    fetch_w(slot, scur);
+    fetch_d(slot, e);
   };
   auto consume = [&](auto slot) __attribute__((always_inline)) {
     constexpr int U = decltype(slot)::value;
@@ -451,48 +520,36 @@ __global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !
 #pragma unroll
       for (int j = 0; j < TY; ++j) acc[i][j] = Op::mma(xf[U][i], y[j], acc[i][j]);
   };
-  // Software pipeline over this wave's k-steps [s0, s1).  Every path issues the same loads in the
+
+  __syncthreads();  // tap table (and the zeroed sums) visible
+
+  // Software pipeline over this wave's k-steps.  Every path issues the same loads in the
   // same (slot) order and only the consumes are conditional, so the wait the compiler places
   // before a consume always leaves the D - 1 younger slots in flight.  (With conditional
   // fetches the wait has to cover the path on which the slot is the youngest load and becomes
   // "wait for everything".)  The price: fetches past the end re-read the last k-step.
   // The sched_barriers keep consume(u) -> fetch(u) in program order; left alone, the scheduler
   // gathers the loads of all D slots at the end of the loop body.
-  auto for_slots = [&](auto f) __attribute__((always_inline)) {
-    f(std::integral_constant<int, 0>{});
-    f(std::integral_constant<int, 1>{});
-    if constexpr (D > 2) f(std::integral_constant<int, 2>{});
-    if constexpr (D > 3) f(std::integral_constant<int, 3>{});
-    if constexpr (D > 4) f(std::integral_constant<int, 4>{});
-    if constexpr (D > 5) f(std::integral_constant<int, 5>{});
-    if constexpr (D > 6) f(std::integral_constant<int, 6>{});
-    if constexpr (D > 7) f(std::integral_constant<int, 7>{});
-  };
-
-  UNIT_TRACE(asm volatile("s_nop 0" ::"v"(xoff[0]), "v"(pixoff[0]), "v"(inside[0])); tr.mark(2);)
-  __syncthreads();  // tap table (and the zeroed sums) visible
-  UNIT_TRACE(tr.mark(3);)
-
-  const int s0 = nsteps * wave / KG, s1 = nsteps * (wave + 1) / KG;
+  // The first round stands outside the loop: the ring was issued weights first, then pixels, and a loop head that
+  // merges that order with the loop's own would make every round wait as if the ring's order still held.
   if (s0 < s1) {
-    sf = s0;
-    slast = s1 - 1;
+    sf = min(s0 + D, slast);
     ecur = tab[kInt ? 2 * sf + half : sf];
-    for_slots([&](auto u) __attribute__((always_inline)) {
-      fetch(u);
-      __builtin_amdgcn_sched_barrier(0);
-    });
-    UNIT_TRACE(tr.mark(4);)
-    int s = s0;
-    // while more than D k-steps remain: consume a round and fetch the next one (in the last round fewer than D
-    // k-steps are new; the surplus fetches repeat the wave's last k-step)
-    for (; s + D < s1; s += D)
+    auto round = [&]() __attribute__((always_inline)) {
       for_slots([&](auto u) __attribute__((always_inline)) {
         consume(u);
         __builtin_amdgcn_sched_barrier(0);
         fetch(u);
         __builtin_amdgcn_sched_barrier(0);
       });
+    };
+    int s = s0;
+    // while more than D k-steps remain: consume a round and fetch the next one (in the last round fewer than D
+    // k-steps are new; the surplus fetches repeat the wave's last k-step)
+    if (s + D < s1) {
+      round();
+      for (s += D; s + D < s1; s += D) round();
+    }
     for_slots([&](auto u) __attribute__((always_inline)) {  // 1 .. D k-steps left, all in flight
       if (s + decltype(u)::value < s1) consume(u);
       __builtin_amdgcn_sched_barrier(0);

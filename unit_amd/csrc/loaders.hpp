@@ -248,6 +248,10 @@ struct ConvGeom {
   // by_plane = by_ohw
   int D, KD, sd, nopad;                 // nopad: no zero padding anywhere (every tap of a valid pixel is inside)
   FastDiv by_plane, by_kd;              // dividers by OH * OW, KD
+  // bit kh * KW set for every window row kh, when the window is undilated and has at most 31 positions (else 0):
+  // the positions of a pixel's window that lie inside the image are then (columns inside) * (these bits of the rows
+  // inside), both of them ranges
+  u32 row_ones;
 };
 
 template <int ROWS, int BKB, int NT, int TAPB, bool XOR80, int PF = 1>

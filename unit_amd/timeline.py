@@ -17,7 +17,7 @@ import sys
 import numpy as np
 
 GEMM_POINTS = ["entry", "ring issued", "stage 0 landed", "last MFMA done", "stores issued", "stores acknowledged"]
-CONV_POINTS = ["entry", "arguments fetched", "tables / window state built", "past the barrier", "ring issued",
+CONV_POINTS = ["entry", "arguments fetched", "weight loads issued", "window state built", "pixel loads issued",
                "reduction done", "k-groups summed", "stores acknowledged"]
 
 
@@ -128,7 +128,8 @@ def main(argv):
                 print(f"   XCD {x}: {len(e)} waves, last MFMA done min {e.min():.2f} median {np.median(e):.2f} max {e.max():.2f}")
         else:
             ph = [(h[:, k + 1].astype(np.int64) - h[:, k].astype(np.int64)) * 0.01 for k in range(7)]
-            names = ["argument fetch", "tables / decode", "barrier", "ring issue", "reduction", "k-group sum", "stores"]
+            names = ["argument fetch", "place + weight loads", "window decode", "tap entries + pixel loads",
+                     "tables, barrier, reduction", "k-group sum", "stores"]
             valid = h[:, 6] > 0
             parts = []
             for k, nm in enumerate(names):
