@@ -252,16 +252,20 @@ __global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !
   auto tap_entry = [&](int e) __attribute__((always_inline)) {
     v2i ent = {0, 31};
     if constexpr (C4) {
-      int rest, kh, ci, kd;
+      int rest, kh;
       g.by_kh.divmod(e >> 1, rest, kh);
-      g.by_kd.divmod(rest, ci, kd);
+      int ci = rest, kd = 0;
+      if (g.KD > 1) g.by_kd.divmod(rest, ci, kd);
       ent[0] = (((ci * g.D + kd) * g.H + kh * g.dh) * g.W) * 4 + (e & 1) * 16;
       ent[1] = g.nopad ? 0 : kh;
     } else if (e < g.ntaps) {
-      int kw, rest, kh, rest2, kd, ci;
-      g.by_kw.divmod(e, rest, kw);
-      g.by_kh.divmod(rest, rest2, kh);
-      g.by_kd.divmod(rest2, ci, kd);
+      // (the dividers by one are skipped: each costs two quarter-rate multiplies on the way to the first loads)
+      int kw = 0, rest = e, kh = 0;
+      if (g.KW > 1) g.by_kw.divmod(e, rest, kw);
+      int rest2 = rest;
+      if (g.KH > 1) g.by_kh.divmod(rest, rest2, kh);
+      int ci = rest2, kd = 0;
+      if (g.KD > 1) g.by_kd.divmod(rest2, ci, kd);
       ent[0] = (((ci * g.D + kd) * g.H + kh * g.dh) * g.W + kw * g.dw) * TAPB;
       ent[1] = g.nopad ? 0 : kh * g.KW + kw;
     }
@@ -335,11 +339,11 @@ __global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !
     for (int i = 0; i < TX; ++i) {
       const u32 o = xoff[i] + xk;
       if constexpr (PREP) {
-        xf[U][i] = *reinterpret_cast<const v4i *>(wgt + xoff[i] + xs);
+        xf[U][i] = *reinterpret_cast<const v4i *>(wgt + (xoff[i] + xs));
       } else if constexpr (C4) {
         const u32 xr = (u32)scur * (u32)(g.KW * 64);  // this k-step's window row
 #pragma unroll
-        for (int d = 0; d < 4; ++d) xf[U][i][d] = *reinterpret_cast<const int *>(wgt + xoff[i] + xr + wtap[d]);
+        for (int d = 0; d < 4; ++d) xf[U][i][d] = *reinterpret_cast<const int *>(wgt + (xoff[i] + xr + wtap[d]));
       } else if constexpr (kInt) {
 #pragma unroll
         for (int d = 0; d < 4; ++d) xf[U][i][d] = *reinterpret_cast<const int *>(wgt + o + d * 64);
@@ -371,9 +375,10 @@ __global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !
     inside[j] = 0;
     if constexpr (C4) colm[j] = v4i{0, 0, 0, 0};
     if (m < g.npix) {
-      int n, rem, od, rem2, oh, ow;
+      int n, rem, oh, ow;
       g.by_ohw.divmod(m, n, rem);
-      g.by_plane.divmod(rem, od, rem2);  // od = 0 for a 2-D convolution
+      int od = 0, rem2 = rem;  // a 2-D convolution
+      if (g.D > 1) g.by_plane.divmod(rem, od, rem2);
       g.by_ow.divmod(rem2, oh, ow);
       const int ih0 = oh * g.sh - g.pt, iw0 = ow * g.sw - g.pl;
       pixoff[j] += (int)(n * g.img_bytes) + ((od * g.sd * g.H + ih0) * g.W + iw0) * TAPB;

@@ -9,6 +9,7 @@ the kernel names, plus shader-clock tick counts; this tool runs the workload in 
 launches first: the clocks of the part follow the load), reads the stamps of the last launch and prints, per
 point, the distribution over the waves relative to the first wave's entry.  The GEMM shapes and operand
 distributions are those of bench.py (4096^3; u8 / s8 uniform, fp16 N(0,1)/64 against N(0,1)).
+UNIT_AMD_TIMELINE_DUMP=<folder> also saves the raw stamps (one row per wave) as <workload>.npy.
 """
 import ctypes
 import os
@@ -104,6 +105,8 @@ def main(argv):
         if len(h) == 0:
             print("   no stamps: this kernel is not instrumented")
             continue
+        if os.environ.get("UNIT_AMD_TIMELINE_DUMP"):  # the raw stamps, one row per wave
+            np.save(os.path.join(os.environ["UNIT_AMD_TIMELINE_DUMP"], what.replace("@", "_at_") + ".npy"), h)
         base = h[:, 0].min()
         last = 0
         for k, name in enumerate(points):
