@@ -83,17 +83,22 @@ def main(argv):
             us = timed(fn, 400)  # the clocks settle after ~300 sustained launches
             points = GEMM_POINTS
         else:
-            match = [s for s in WL.RESNET50 if s.name == what and s.C % 16 == 0]
+            match = [s for s in WL.RESNET50 if s.name == what]
             if not match:
                 sys.exit(f"unknown workload {what!r}")
             s = match[0]
-            data = t(rng.uniform_u8((batch, s.C // 16, s.H, s.W, 16), 1))
-            wt = U.prepack_conv_weight(t(rng.uniform_s8((s.K, s.C, s.KH, s.KW), 2)), 16)
+            cb = WL.channel_block(s.C)  # 4 for the three-channel stem (padded input channels hold zeros)
+            cp = -(-s.C // cb) * cb
+            data_np = rng.uniform_u8((batch, cp // cb, s.H, s.W, cb), 1)
+            if cp != s.C:
+                data_np[..., s.C % cb:] = 0
+            data = t(data_np)
+            wt = U.prepack_conv_weight(t(rng.uniform_s8((s.K, s.C, s.KH, s.KW), 2)), cb)
             prep = U.prepare_conv2d_weight(wt)
             oh, ow = WL.out_hw(s)
             out = torch.empty((batch, s.K // 16, oh, ow, 16), dtype=torch.int32, device=dev)
-            desc = _lib.ConvDesc(batch, s.C, s.H, s.W, s.K, s.KH, s.KW, s.stride, s.stride, s.pad, s.pad, s.pad, s.pad,
-                                 1, 1, 16)
+            desc = _lib.ConvDesc(batch, cp, s.H, s.W, s.K, s.KH, s.KW, s.stride, s.stride, s.pad, s.pad, s.pad, s.pad,
+                                 1, 1, cb)
             fn = lambda: _lib.check(L.unit_conv2d_nchwc_u8s8s32_prepared(ctypes.byref(desc), data.data_ptr(),
                                                                          prep.buf.data_ptr(), out.data_ptr(), stream))
             us = timed(fn, 10)
@@ -106,6 +111,7 @@ def main(argv):
             print("   no stamps: this kernel is not instrumented")
             continue
         if os.environ.get("UNIT_AMD_TIMELINE_DUMP"):  # the raw stamps, one row per wave
+            os.makedirs(os.environ["UNIT_AMD_TIMELINE_DUMP"], exist_ok=True)
             np.save(os.path.join(os.environ["UNIT_AMD_TIMELINE_DUMP"], what.replace("@", "_at_") + ".npy"), h)
         base = h[:, 0].min()
         last = 0
