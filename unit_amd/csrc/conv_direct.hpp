@@ -468,8 +468,11 @@ __global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !
       }
     }
   }
-  // the tap table for the fetches after the ring, and the zeroed sums
-  for (int e = threadIdx.x; e < ntab; e += S::NT) tab[e] = tap_entry(e);
+  // the tap table for the fetches after the ring -- not built, and its barrier not taken, when no wave of the
+  // workgroup has more k-steps than the ring holds -- and the zeroed sums
+  const bool need_tab = (nsteps + KG - 1) / KG > D;
+  if (need_tab)
+    for (int e = threadIdx.x; e < ntab; e += S::NT) tab[e] = tap_entry(e);
   if constexpr (KG > 1 && !kParked) {
     v4i *z = reinterpret_cast<v4i *>(tiles);
     for (int e = threadIdx.x; e < (S::TILE + S::WSUM) / 16; e += S::NT) z[e] = v4i{0, 0, 0, 0};
@@ -526,7 +529,7 @@ __global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !
       for (int j = 0; j < TY; ++j) acc[i][j] = Op::mma(xf[U][i], y[j], acc[i][j]);
   };
 
-  __syncthreads();  // tap table (and the zeroed sums) visible
+  if (need_tab) __syncthreads();  // tap table (and the zeroed sums) visible
 
   // Software pipeline over this wave's k-steps.  Every path issues the same loads in the
   // same (slot) order and only the consumes are conditional, so the wait the compiler places
@@ -539,7 +542,7 @@ __global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !
   // merges that order with the loop's own would make every round wait as if the ring's order still held.
   if (s0 < s1) {
     sf = min(s0 + D, slast);
-    ecur = tab[kInt ? 2 * sf + half : sf];
+    if (need_tab) ecur = tab[kInt ? 2 * sf + half : sf];
     auto round = [&]() __attribute__((always_inline)) {
       for_slots([&](auto u) __attribute__((always_inline)) {
         consume(u);
@@ -589,6 +592,7 @@ __global__ __launch_bounds__(S::NT) __attribute__((amdgpu_waves_per_eu(PREP && !
                           scratch);
   } else if constexpr (!kParked) {
     // sum the partial tiles of the KG waves in LDS, then share the blocks among the waves
+    if (!need_tab) __syncthreads();  // the zeroed sums, when the barrier before the reduction was not taken
     int *sum = reinterpret_cast<int *>(tiles);
 #pragma unroll
     for (int i = 0; i < TX; ++i)
