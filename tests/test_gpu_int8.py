@@ -156,6 +156,10 @@ CONV_CASES = [
     (32, 256, 14, 14, 256, 3, 1, 1, 1),    # batch 32: 256-channel tile
     (32, 128, 28, 28, 128, 3, 1, 1, 1),    # batch 32: 128-channel tile
     (8, 512, 7, 7, 2048, 1, 1, 0, 1),
+    (1, 16, 5, 5, 32, 3, 1, 3, 1),         # padding as wide as the window: border windows lie outside altogether
+    (2, 32, 2, 3, 32, 3, 1, 1, 1),         # image smaller than the window: cut on both sides at once
+    (1, 16, 3, 3, 16, 5, 1, 2, 1),         # 5x5 on 3x3: every window loses rows and columns at both ends
+    (2, 32, 6, 9, 32, 3, 2, (2, 0, 1, 3), 1),   # stride 2, four different pads
 ]
 
 
