@@ -411,6 +411,13 @@ def main():
     us_fp = time_us(g_fp, 30, warm=GEMM_WARM, bursts=3)
     v_fp, min_fp = U.last_variant(), last_min[0]
 
+    # fp16 output (BASELINE.json configs[2] names both output types; the reference script's own result is fp32,
+    # apps/gpu/gemm.py:14-20): half the bytes to write back
+    ch = torch.empty((M, N), dtype=torch.float16, device=dev)
+    g_fh = lambda: _lib.check(L.unit_gemm_f16(ah.data_ptr(), bh.data_ptr(), ch.data_ptr(), M, N, K, 1, stream))
+    us_fh = time_us(g_fh, 30, warm=GEMM_WARM, bursts=3)
+    v_fh, min_fh = U.last_variant(), last_min[0]
+
     def f16_err():  # every 16th row of the result against float64
         torch.cuda.synchronize()
         ref = ah_np[::16].astype(np.float64) @ bh_np.astype(np.float64)
@@ -420,13 +427,22 @@ def main():
     err_f = f16_err()
     g_fp()
     err_fp = f16_err()
+    g_fh()
+    torch.cuda.synchronize()
+    ref_h = ah_np[::16].astype(np.float64) @ bh_np.astype(np.float64)
+    got_h = ch[::16].float().cpu().numpy().astype(np.float64)
+    err_fh = float((np.abs(got_h - ref_h) / np.maximum(np.abs(ref_h), 1e-3 * np.abs(ref_h).max())).max())
+    del ch, ref_h, got_h
     gemm_f16 = dict(workload="fp16 GEMM 4096^3, fp32 accumulate, fp32 out", timing=gemm_timing,
                     us=round(us_f, 2), us_min=round(min_f, 2), tflops=round(gemm_ops / us_f / 1e6, 1),
                     pct_f16_peak=round(100 * gemm_ops / us_f / 1e6 / PEAK_F16_TFLOPS, 2), kernel=v_f,
                     max_rel_err=err_f, tolerance=1e-2, rows_checked=M // 16,
                     prepared_b=dict(us=round(us_fp, 2), us_min=round(min_fp, 2), tflops=round(gemm_ops / us_fp / 1e6, 1),
                                     pct_f16_peak=round(100 * gemm_ops / us_fp / 1e6 / PEAK_F16_TFLOPS, 2), kernel=v_fp,
-                                    max_rel_err=err_fp))
+                                    max_rel_err=err_fp),
+                    f16_out=dict(us=round(us_fh, 2), us_min=round(min_fh, 2), tflops=round(gemm_ops / us_fh / 1e6, 1),
+                                 pct_f16_peak=round(100 * gemm_ops / us_fh / 1e6 / PEAK_F16_TFLOPS, 2), kernel=v_fh,
+                                 max_rel_err=err_fh))
 
     # the reference's own GEMM sizes (its drivers' constants): few output tiles, so the reduction is split between workgroups
     ra = torch.randint(0, 256, (128, 768), dtype=torch.uint8, device=dev)
@@ -739,7 +755,8 @@ def main():
         "gemm_fp16_pct_peak": gemm_f16["pct_f16_peak"],
         "gemm_fp16_prepared_b_us": gemm_f16["prepared_b"]["us"],
         "gemm_fp16_prepared_b_pct_peak": gemm_f16["prepared_b"]["pct_f16_peak"],
-        "gemm_fp16_max_rel_err": round(max(err_f, err_fp), 6),
+        "gemm_fp16_f16_out_us": gemm_f16["f16_out"]["us"],
+        "gemm_fp16_max_rel_err": round(max(err_f, err_fp, err_fh), 6),
         "sum_layers_cold_us": round(sum(ly["us_cold"] * ly["shape"].count for ly in layers), 1),
         "launch": launch_mode,
         "fp16_conv": dict(stack_us=conv_fp16["stack_us"], tflops=conv_fp16["tflops"]),
